@@ -1,0 +1,85 @@
+// Shared host/device helpers of the FlashMoE gfx950 kernels: status + error text, element-type
+// traits, wave64 reductions.  Everything here targets CDNA4 only (64-lane wavefronts).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/flashmoe_hip.h"
+
+namespace fmoe {
+
+constexpr int kWave = 64;
+
+// ---- error reporting -------------------------------------------------------------------------
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+
+#define FMOE_REQUIRE(cond, status, ...)          \
+    do {                                         \
+        if (!(cond)) {                           \
+            ::fmoe::set_error(__VA_ARGS__);      \
+            return (status);                     \
+        }                                        \
+    } while (0)
+
+// Launch check: hipGetLastError after a launch; returns the positive hipError_t on failure.
+#define FMOE_CHECK_LAUNCH(what)                                                        \
+    do {                                                                               \
+        hipError_t e__ = hipGetLastError();                                            \
+        if (e__ != hipSuccess) {                                                       \
+            ::fmoe::set_error("%s: launch failed: %s", what, hipGetErrorString(e__));  \
+            return (int)e__;                                                           \
+        }                                                                              \
+    } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline size_t dtype_size(int dtype) { return dtype == FMOE_F32 ? 4 : 2; }
+inline bool dtype_ok(int dtype) { return dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16; }
+inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// ---- element types ---------------------------------------------------------------------------
+using bf16_t = __bf16;
+using f16_t = _Float16;
+
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int kVec = 4;   // elements per 16-byte load
+    __device__ static float to_f32(float v) { return v; }
+    __device__ static float from_f32(float v) { return v; }
+};
+template <> struct Elem<bf16_t> {
+    static constexpr int kVec = 8;
+    __device__ static float to_f32(bf16_t v) { return (float)v; }
+    __device__ static bf16_t from_f32(float v) { return (bf16_t)v; }
+};
+template <> struct Elem<f16_t> {
+    static constexpr int kVec = 8;
+    __device__ static float to_f32(f16_t v) { return (float)v; }
+    __device__ static f16_t from_f32(float v) { return (f16_t)v; }
+};
+
+// Round an fp32 value to T and back (what "computed in the input dtype" means for one add).
+template <typename T> __device__ inline float round_through(float v) { return Elem<T>::to_f32(Elem<T>::from_f32(v)); }
+
+// ---- wave64 helpers --------------------------------------------------------------------------
+__device__ inline int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+    return v;
+}
+
+__device__ inline float silu_f32(float v) { return v / (1.0f + __expf(-v)); }
+
+}  // namespace fmoe

@@ -1,0 +1,343 @@
+// Shared SwiGLU MLP for gfx950:  out = (silu(x Wg^T) * (x Wu^T)) Wd^T [+ residual]
+//
+// Two launches of one MFMA GEMM kernel  C[M,N] = A[M,K] * B[N,K]^T  (both operands K-contiguous, which
+// is how x, the nn.Linear weights and the [T,I] activation are laid out, so a lane's 8 consecutive k
+// values for v_mfma_f32_32x32x16 are one 16-byte LDS read):
+//   1. gate/up: the B tile holds BN/2 rows of Wg and the same BN/2 rows of Wu, so each wave owns
+//      matching gate and up accumulators and the epilogue writes silu(gate)*up, rounded once, to the
+//      [T,I] workspace.  The gate and up products never go to memory.
+//   2. down: plain epilogue, optional residual add (the routed-expert output in the block).
+// 256 threads = 4 waves in a 2x2 arrangement, each wave (BM/2)x(BN/2) of 32x32 MFMA tiles; A and B tiles
+// go global -> registers -> LDS with the next tile's global loads issued before the current tile's
+// MFMAs; LDS rows are 128 bytes with the 16-byte chunk index XOR-ed with (row & 7) so that the 32 rows
+// a fragment read touches spread over all banks.  Workgroup ids are remapped so that each XCD (ids are
+// dealt round-robin over the 8 XCDs) works on a compact patch of the tile grid and shares A/B tiles in
+// its own L2.
+#include "fmoe_common.h"
+
+namespace fmoe {
+namespace {
+
+constexpr int kGemmThreads = 256;
+constexpr int BK = 64;            // k extent of an LDS tile (elements); 8 chunks of 8 elements per row
+constexpr int kChunksPerRow = BK / 8;
+
+enum Epilogue { kEpiSwiGLU = 0, kEpiPlain = 1 };
+
+template <typename T> struct Mfma32;
+template <> struct Mfma32<bf16_t> {
+    using Frag = bf16x8_t;
+    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mfma32<f16_t> {
+    using Frag = f16x8_t;
+    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+__device__ inline int swizzled_offset(int row, int chunk) {   // element offset inside a [rows][BK] tile
+    return row * BK + ((chunk ^ (row & 7)) << 3);
+}
+
+// Map the linear workgroup id to a tile so that each XCD gets a contiguous run of the tile order, and
+// the tile order walks GM tile-rows at a time (compact patches share A and B tiles).
+__device__ inline void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int nb = (int)gridDim.x;
+    int t = (int)blockIdx.x;
+    if ((nb & 7) == 0) t = (t & 7) * (nb >> 3) + (t >> 3);
+    constexpr int GM = 8;
+    const int width = GM * tiles_n;
+    const int group = t / width;
+    const int first_m = group * GM;
+    const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+    tm = first_m + (t % width) % gsz;
+    tn = (t % width) / gsz;
+}
+
+template <typename T, int BM, int BN, int EPI>
+__global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
+    const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
+    const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n) {
+    using Frag = typename Mfma32<T>::Frag;
+    constexpr int WM = BM / 2, WN = BN / 2;        // per-wave tile
+    constexpr int MF = WM / 32, NF = WN / 32;      // 32x32 fragments per wave
+    constexpr int A_CHUNKS = BM * kChunksPerRow / kGemmThreads;
+    constexpr int B_CHUNKS = BN * kChunksPerRow / kGemmThreads;
+    constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;   // output columns per tile
+
+    __shared__ __attribute__((aligned(16))) T As[BM * BK];
+    __shared__ __attribute__((aligned(16))) T Bs[BN * BK];
+
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN_OUT;
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    u32x4_t ra[A_CHUNKS], rb[B_CHUNKS];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < A_CHUNKS; ++it) {
+            const int q = it * kGemmThreads + tid;
+            const int row = q / kChunksPerRow, ch = q % kChunksPerRow;
+            const int gm = m0 + row, gk = k0 + ch * 8;
+            ra[it] = (gm < M && gk < K) ? *reinterpret_cast<const u32x4_t*>(A + (int64_t)gm * K + gk) : zero4;
+        }
+#pragma unroll
+        for (int it = 0; it < B_CHUNKS; ++it) {
+            const int q = it * kGemmThreads + tid;
+            const int row = q / kChunksPerRow, ch = q % kChunksPerRow;
+            const int gk = k0 + ch * 8;
+            const T* base;
+            int gn;
+            if (EPI == kEpiSwiGLU) {
+                const bool is_up = row >= BN / 2;
+                base = is_up ? B1 : B0;
+                gn = n0 + (is_up ? row - BN / 2 : row);
+            } else {
+                base = B0;
+                gn = n0 + row;
+            }
+            rb[it] = (gn < N && gk < K) ? *reinterpret_cast<const u32x4_t*>(base + (int64_t)gn * K + gk) : zero4;
+        }
+    };
+    auto store_lds = [&]() {
+#pragma unroll
+        for (int it = 0; it < A_CHUNKS; ++it) {
+            const int q = it * kGemmThreads + tid;
+            *reinterpret_cast<u32x4_t*>(&As[swizzled_offset(q / kChunksPerRow, q % kChunksPerRow)]) = ra[it];
+        }
+#pragma unroll
+        for (int it = 0; it < B_CHUNKS; ++it) {
+            const int q = it * kGemmThreads + tid;
+            *reinterpret_cast<u32x4_t*>(&Bs[swizzled_offset(q / kChunksPerRow, q % kChunksPerRow)]) = rb[it];
+        }
+    };
+
+    f32x16_t acc[MF][NF];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int j = 0; j < NF; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // LDS row of this lane inside fragment f of the wave's A / B sub-tile
+    const int frag_row = lane & 31;
+    const int frag_half = lane >> 5;   // which 8 of the 16 k values of one MFMA this lane supplies
+    int b_row[NF];
+#pragma unroll
+    for (int j = 0; j < NF; ++j) {
+        if (EPI == kEpiSwiGLU)
+            b_row[j] = (j < NF / 2) ? wn * (BN / 4) + j * 32 + frag_row
+                                    : BN / 2 + wn * (BN / 4) + (j - NF / 2) * 32 + frag_row;
+        else
+            b_row[j] = wn * WN + j * 32 + frag_row;
+    }
+
+    const int k_tiles = (K + BK - 1) / BK;
+    load_global(0);
+    store_lds();
+    __syncthreads();
+
+    for (int kt = 0; kt < k_tiles; ++kt) {
+        if (kt + 1 < k_tiles) load_global((kt + 1) * BK);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            const int chunk = ks * 2 + frag_half;
+            Frag fa[MF], fb[NF];
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+                fa[i] = *reinterpret_cast<const Frag*>(&As[swizzled_offset(wm * WM + i * 32 + frag_row, chunk)]);
+#pragma unroll
+            for (int j = 0; j < NF; ++j) fb[j] = *reinterpret_cast<const Frag*>(&Bs[swizzled_offset(b_row[j], chunk)]);
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+                for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[i], fb[j], acc[i][j]);
+        }
+        __syncthreads();
+        if (kt + 1 < k_tiles) {
+            store_lds();
+            __syncthreads();
+        }
+    }
+
+    // D fragment layout of v_mfma_f32_32x32x*: lane l, register v holds
+    //   row = 8*(v/4) + 4*(l/32) + (v%4)   (A / M index),   col = l%32   (B / N index)
+    if (EPI == kEpiSwiGLU) {
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int j = 0; j < NF / 2; ++j) {
+                const int col = n0 + wn * (BN / 4) + j * 32 + frag_row;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * frag_half + (v % 4);
+                    if (row < M && col < N) {
+                        const float g = acc[i][j][v], u = acc[i][j + NF / 2][v];
+                        C[(int64_t)row * N + col] = Elem<T>::from_f32(silu_f32(g) * u);
+                    }
+                }
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int j = 0; j < NF; ++j) {
+                const int col = n0 + wn * WN + j * 32 + frag_row;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * frag_half + (v % 4);
+                    if (row < M && col < N) {
+                        float r = acc[i][j][v];
+                        if (R != nullptr) r += Elem<T>::to_f32(R[(int64_t)row * N + col]);
+                        C[(int64_t)row * N + col] = Elem<T>::from_f32(r);
+                    }
+                }
+            }
+    }
+}
+
+// fp32 path (parity configuration only; not a tuned kernel): 64x64 tile, 16-deep LDS slabs, 4x4 outputs
+// per thread, plain FMA.
+template <int EPI>
+__global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__ A, const float* __restrict__ B0,
+                                                       const float* __restrict__ B1, float* __restrict__ C,
+                                                       const float* __restrict__ R, int M, int N, int K) {
+    constexpr int TS = 64, KS = 16;
+    __shared__ float As[KS][TS + 1];
+    __shared__ float Bg[KS][TS + 1];
+    __shared__ float Bu[(EPI == kEpiSwiGLU) ? KS : 1][TS + 1];
+    const int m0 = blockIdx.y * TS, n0 = blockIdx.x * TS;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    float accg[4][4] = {}, accu[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += KS) {
+        for (int q = threadIdx.x; q < TS * KS; q += 256) {
+            const int r = q / KS, kk = q % KS;
+            const int gk = k0 + kk;
+            As[kk][r] = (m0 + r < M && gk < K) ? A[(int64_t)(m0 + r) * K + gk] : 0.0f;
+            Bg[kk][r] = (n0 + r < N && gk < K) ? B0[(int64_t)(n0 + r) * K + gk] : 0.0f;
+            if (EPI == kEpiSwiGLU) Bu[kk][r] = (n0 + r < N && gk < K) ? B1[(int64_t)(n0 + r) * K + gk] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            float a[4], g[4], u[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                g[j] = Bg[kk][tx * 4 + j];
+                u[j] = (EPI == kEpiSwiGLU) ? Bu[kk][tx * 4 + j] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    accg[i][j] = __builtin_fmaf(a[i], g[j], accg[i][j]);
+                    if (EPI == kEpiSwiGLU) accu[i][j] = __builtin_fmaf(a[i], u[j], accu[i][j]);
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = m0 + ty * 4 + i, col = n0 + tx * 4 + j;
+            if (row < M && col < N) {
+                float r = (EPI == kEpiSwiGLU) ? silu_f32(accg[i][j]) * accu[i][j] : accg[i][j];
+                if (EPI == kEpiPlain && R != nullptr) r += R[(int64_t)row * N + col];
+                C[(int64_t)row * N + col] = r;
+            }
+        }
+}
+
+template <typename T, int BM, int BN, int EPI>
+void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
+    constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_OUT - 1) / BN_OUT;
+    hipLaunchKernelGGL((gemm_nt_kernel<T, BM, BN, EPI>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), 0,
+                       stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
+}
+
+template <typename T>
+int mlp_16bit(const void* x, const void* wg, const void* wu, const void* wd, int64_t T_, int H, int I,
+              const void* residual, void* out, void* h, hipStream_t stream) {
+    const int M = (int)T_;
+    // gate/up: N = I output columns; down: N = H.  Large tiles when they still give every CU work.
+    const int64_t big_tiles_1 = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
+    if (big_tiles_1 >= 256)
+        launch_gemm<T, 256, 256, kEpiSwiGLU>((const T*)x, (const T*)wg, (const T*)wu, (T*)h, nullptr, M, I, H, stream);
+    else
+        launch_gemm<T, 128, 128, kEpiSwiGLU>((const T*)x, (const T*)wg, (const T*)wu, (T*)h, nullptr, M, I, H, stream);
+    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(gate/up)");
+    const int64_t big_tiles_2 = (int64_t)((M + 255) / 256) * ((H + 255) / 256);
+    if (big_tiles_2 >= 256)
+        launch_gemm<T, 256, 256, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
+    else
+        launch_gemm<T, 128, 128, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
+    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(down)");
+    return FMOE_OK;
+}
+
+int mlp_f32(const void* x, const void* wg, const void* wu, const void* wd, int64_t T_, int H, int I,
+            const void* residual, void* out, void* h, hipStream_t stream) {
+    const int M = (int)T_;
+    hipLaunchKernelGGL((sgemm_nt_kernel<kEpiSwiGLU>), dim3((I + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
+                       (const float*)x, (const float*)wg, (const float*)wu, (float*)h, nullptr, M, I, H);
+    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(gate/up, f32)");
+    hipLaunchKernelGGL((sgemm_nt_kernel<kEpiPlain>), dim3((H + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
+                       (const float*)h, (const float*)wd, nullptr, (float*)out, (const float*)residual, M, H, I);
+    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(down, f32)");
+    return FMOE_OK;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" size_t fmoe_mlp_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int dtype) {
+    (void)hidden;
+    if (num_tokens <= 0 || intermediate <= 0 || !fmoe::dtype_ok(dtype)) return 0;
+    return fmoe::round_up((size_t)num_tokens * (size_t)intermediate * fmoe::dtype_size(dtype), 256);
+}
+
+extern "C" int fmoe_mlp_forward(const void* x, const void* gate_w, const void* up_w, const void* down_w,
+                                int64_t num_tokens, int hidden, int intermediate, int dtype, const void* residual,
+                                void* out, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_mlp_forward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && intermediate > 0, FMOE_ERR_BAD_SHAPE,
+                 "fmoe_mlp_forward: bad shape T=%lld H=%d I=%d", (long long)num_tokens, hidden, intermediate);
+    FMOE_REQUIRE(num_tokens < (1ll << 31), FMOE_ERR_UNSUPPORTED, "fmoe_mlp_forward: T=%lld >= 2^31",
+                 (long long)num_tokens);
+    if (num_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(x && gate_w && up_w && down_w && out, FMOE_ERR_NULL_POINTER, "fmoe_mlp_forward: null tensor pointer");
+    const size_t need = fmoe_mlp_workspace_bytes(num_tokens, hidden, intermediate, dtype);
+    FMOE_REQUIRE(workspace && workspace_bytes >= need, FMOE_ERR_WORKSPACE,
+                 "fmoe_mlp_forward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    if (dtype != FMOE_F32) {
+        FMOE_REQUIRE(hidden % 8 == 0 && intermediate % 8 == 0, FMOE_ERR_ALIGNMENT,
+                     "fmoe_mlp_forward: hidden=%d and intermediate=%d must be multiples of 8 (16-byte rows)", hidden,
+                     intermediate);
+        FMOE_REQUIRE(aligned16(x) && aligned16(gate_w) && aligned16(up_w) && aligned16(down_w) && aligned16(workspace),
+                     FMOE_ERR_ALIGNMENT, "fmoe_mlp_forward: tensor pointers must be 16-byte aligned");
+    }
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FMOE_F32: return mlp_f32(x, gate_w, up_w, down_w, num_tokens, hidden, intermediate, residual, out, workspace, s);
+        case FMOE_BF16: return mlp_16bit<bf16_t>(x, gate_w, up_w, down_w, num_tokens, hidden, intermediate, residual, out, workspace, s);
+        default: return mlp_16bit<f16_t>(x, gate_w, up_w, down_w, num_tokens, hidden, intermediate, residual, out, workspace, s);
+    }
+}

@@ -1,0 +1,245 @@
+// Product-key router for gfx950: per token, the K largest sums a[i] + b[j] over two score vectors
+// of nk entries each, without materialising the nk*nk sums.
+//
+// Exact pruning.  Order each half by (score descending, key index ascending) and call the rank of
+// an entry in that order r.  A pair of ranks (ri, rj) is dominated by the (ri+1)*(rj+1)-1 pairs whose
+// ranks are component-wise <=, because fp32 addition is monotone in each operand.  So only pairs with
+// (ri+1)*(rj+1) <= K can be among the K best: sum_i floor(K/i) candidates (280 for K=64, 645 for
+// K=128) instead of nk*nk (16384 / 262144).  The returned scores are therefore exactly the K largest
+// sums; where sums tie exactly at the cut the chosen index may differ from an exhaustive scan.
+//
+// One wavefront handles one token.  All selection is done with 64-bit keys
+//   (order-preserving bits of the fp32 score) << 32 | ~index
+// so that "larger key" means "larger score, then smaller index".  top-K of a long list is computed in
+// groups of KP = max(64, next_pow2(K)) keys: each group is bitonic-sorted across the wave (RK = KP/64
+// keys per lane), odd groups in ascending order so that max(best[p], group[p]) is the bitonic sequence
+// holding the K best of both, which one bitonic merge re-sorts.
+#include <math.h>
+
+#include "fmoe_common.h"
+
+namespace fmoe {
+namespace {
+
+constexpr int kRouterWaves = 4;
+constexpr int kMaxTopK = 256;
+constexpr int kMaxCand = 2048;   // >= sum_{i=1..256} floor(256/i) = 1546
+
+__device__ inline uint32_t order_bits(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+__device__ inline float order_value(uint32_t o) {
+    return __uint_as_float(o ^ ((o >> 31) ? 0x80000000u : 0xffffffffu));
+}
+__device__ inline uint64_t make_key(float score, uint32_t index) {
+    return ((uint64_t)order_bits(score) << 32) | (uint64_t)(~index);
+}
+__device__ inline float key_score(uint64_t k) { return order_value((uint32_t)(k >> 32)); }
+__device__ inline uint32_t key_index(uint64_t k) { return ~(uint32_t)(k & 0xffffffffu); }
+
+__device__ inline uint64_t shfl_xor_u64(uint64_t v, int mask) {
+    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, kWave);
+    const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, kWave);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// Position of a key in the wave-wide sequence: p = lane*RK + r.
+// One compare-exchange layer of a bitonic network: partner = p ^ j, blocks of size k alternate direction.
+template <int RK, bool DESC>
+__device__ inline void bitonic_layer(uint64_t (&v)[RK], int lane, int k, int j) {
+    if (j < RK) {
+#pragma unroll
+        for (int r = 0; r < RK; ++r) {
+            if ((r & j) == 0) {
+                const int p = lane * RK + r;
+                const bool desc_block = (((p & k) == 0) == DESC);
+                const uint64_t a = v[r], b = v[r | j];
+                const uint64_t hi = a > b ? a : b, lo = a > b ? b : a;
+                v[r] = desc_block ? hi : lo;
+                v[r | j] = desc_block ? lo : hi;
+            }
+        }
+    } else {
+        const int m = j / RK;
+#pragma unroll
+        for (int r = 0; r < RK; ++r) {
+            const int p = lane * RK + r;
+            const uint64_t other = shfl_xor_u64(v[r], m);
+            const bool desc_block = (((p & k) == 0) == DESC);
+            const bool first = (p & j) == 0;
+            const bool keep_max = (first == desc_block);
+            const uint64_t mx = v[r] > other ? v[r] : other;
+            const uint64_t mn = v[r] > other ? other : v[r];
+            v[r] = keep_max ? mx : mn;
+        }
+    }
+}
+
+template <int RK, bool DESC>
+__device__ inline void bitonic_sort(uint64_t (&v)[RK], int lane) {
+    constexpr int N = RK * kWave;
+#pragma unroll
+    for (int k = 2; k <= N; k <<= 1)
+#pragma unroll
+        for (int j = k >> 1; j >= 1; j >>= 1) bitonic_layer<RK, DESC>(v, lane, k, j);
+}
+
+// v holds a bitonic sequence of N keys; sort it descending.
+template <int RK>
+__device__ inline void bitonic_merge_desc(uint64_t (&v)[RK], int lane) {
+    constexpr int N = RK * kWave;
+#pragma unroll
+    for (int j = N >> 1; j >= 1; j >>= 1) bitonic_layer<RK, true>(v, lane, N, j);
+}
+
+// Fold one more group of KP keys into the running sorted-descending top-KP.
+template <int RK, typename Gen>
+__device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_groups, Gen gen) {
+    {
+        uint64_t cur[RK];
+#pragma unroll
+        for (int r = 0; r < RK; ++r) cur[r] = gen(0, r);
+        bitonic_sort<RK, true>(cur, lane);
+#pragma unroll
+        for (int r = 0; r < RK; ++r) best[r] = cur[r];
+    }
+    for (int g = 1; g < num_groups; ++g) {
+        uint64_t cur[RK];
+#pragma unroll
+        for (int r = 0; r < RK; ++r) cur[r] = gen(g, r);
+        bitonic_sort<RK, false>(cur, lane);
+#pragma unroll
+        for (int r = 0; r < RK; ++r) best[r] = best[r] > cur[r] ? best[r] : cur[r];
+        bitonic_merge_desc<RK>(best, lane);
+    }
+}
+
+template <typename T, int RK>
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
+    const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
+    int64_t* __restrict__ indices, T* __restrict__ gates, int norm_topk_prob) {
+    constexpr int KP = RK * kWave;
+    __shared__ uint16_t cand[kMaxCand];
+    __shared__ float half_score[kRouterWaves][2][KP];
+    __shared__ uint32_t half_index[kRouterWaves][2][KP];
+
+    // candidate table: all (i, j) with (i+1)*(j+1) <= K, packed i | j << 8
+    for (int i = threadIdx.x; i < top_k; i += blockDim.x) {
+        int off = 0;
+        for (int q = 0; q < i; ++q) off += top_k / (q + 1);
+        const int n = top_k / (i + 1);
+        for (int j = 0; j < n; ++j) cand[off + j] = (uint16_t)(i | (j << 8));
+    }
+    __syncthreads();
+
+    const int lane = lane_id();
+    const int wave = (int)(threadIdx.x >> 6);
+    const int64_t waves_total = (int64_t)gridDim.x * kRouterWaves;
+    const int64_t rounds = (num_tokens + waves_total - 1) / waves_total;
+    const int half_groups = (nk + KP - 1) / KP;
+    const int cand_groups = (num_cand + KP - 1) / KP;
+
+    for (int64_t round = 0; round < rounds; ++round) {
+        const int64_t token = round * waves_total + (int64_t)blockIdx.x * kRouterWaves + wave;
+        const bool active = token < num_tokens;
+        if (active) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const T* row = lp + ((int64_t)h * num_tokens + token) * nk;
+                uint64_t best[RK];
+                topk_groups<RK>(best, lane, half_groups, [&](int g, int r) -> uint64_t {
+                    const int p = g * KP + lane * RK + r;
+                    return p < nk ? make_key(Elem<T>::to_f32(row[p]), (uint32_t)p) : 0ull;
+                });
+#pragma unroll
+                for (int r = 0; r < RK; ++r) {
+                    half_score[wave][h][lane * RK + r] = key_score(best[r]);
+                    half_index[wave][h][lane * RK + r] = key_index(best[r]);
+                }
+            }
+        }
+        __syncthreads();
+        if (active) {
+            uint64_t best[RK];
+            topk_groups<RK>(best, lane, cand_groups, [&](int g, int r) -> uint64_t {
+                const int c = g * KP + lane * RK + r;
+                if (c >= num_cand) return 0ull;
+                const int ij = cand[c];
+                const int i = ij & 0xff, j = ij >> 8;
+                const float s = round_through<T>(half_score[wave][0][i] + half_score[wave][1][j]);
+                const uint32_t flat = half_index[wave][0][i] * (uint32_t)nk + half_index[wave][1][j];
+                return make_key(s, flat);
+            });
+            float e[RK];
+            float total = 0.0f;
+#pragma unroll
+            for (int r = 0; r < RK; ++r) {
+                const int p = lane * RK + r;
+                e[r] = p < top_k ? expf(key_score(best[r])) : 0.0f;
+                total += e[r];
+            }
+            if (gates != nullptr && norm_topk_prob) total = wave_sum(total);
+#pragma unroll
+            for (int r = 0; r < RK; ++r) {
+                const int p = lane * RK + r;
+                if (p < top_k) {
+                    const int64_t o = token * top_k + p;
+                    scores[o] = Elem<T>::from_f32(key_score(best[r]));
+                    indices[o] = (int64_t)key_index(best[r]);
+                    if (gates != nullptr) gates[o] = Elem<T>::from_f32(norm_topk_prob ? e[r] / total : e[r]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+int count_candidates(int top_k) {
+    int n = 0;
+    for (int i = 1; i <= top_k; ++i) n += top_k / i;
+    return n;
+}
+
+template <typename T>
+int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64_t* indices, void* gates,
+                  int norm, hipStream_t stream) {
+    const int num_cand = count_candidates(K);
+    const int64_t blocks_needed = (T_ + kRouterWaves - 1) / kRouterWaves;
+    const int64_t max_blocks = 256 * 8;   // a few resident blocks per CU; the kernel loops over tokens
+    const dim3 grid((unsigned)(blocks_needed < max_blocks ? blocks_needed : max_blocks));
+    const dim3 block(kRouterWaves * kWave);
+#define FMOE_LAUNCH_ROUTER(R)                                                                                \
+    hipLaunchKernelGGL((router_topk_kernel<T, R>), grid, block, 0, stream, (const T*)lp, T_, nk, K, num_cand, \
+                       (T*)scores, indices, (T*)gates, norm)
+    if (K <= 64) FMOE_LAUNCH_ROUTER(1);
+    else if (K <= 128) FMOE_LAUNCH_ROUTER(2);
+    else FMOE_LAUNCH_ROUTER(4);
+#undef FMOE_LAUNCH_ROUTER
+    FMOE_CHECK_LAUNCH("fmoe_router_topk");
+    return FMOE_OK;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
+                                void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_router_topk: unknown dtype %d", dtype);
+    FMOE_REQUIRE(num_tokens >= 0 && num_keys > 0, FMOE_ERR_BAD_SHAPE, "fmoe_router_topk: bad shape T=%lld nk=%d",
+                 (long long)num_tokens, num_keys);
+    FMOE_REQUIRE(top_k >= 0 && top_k <= num_keys, FMOE_ERR_TOPK_RANGE,
+                 "num_experts_per_tok should be in [0, %d], but got %d", num_keys, top_k);
+    FMOE_REQUIRE(num_keys <= 65535, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk: num_keys=%d > 65535", num_keys);
+    FMOE_REQUIRE(top_k <= kMaxTopK, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk: top_k=%d > %d", top_k, kMaxTopK);
+    if (num_tokens == 0 || top_k == 0) return FMOE_OK;
+    FMOE_REQUIRE(log_probs && scores && indices, FMOE_ERR_NULL_POINTER, "fmoe_router_topk: null tensor pointer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FMOE_F32: return launch_router<float>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+        case FMOE_BF16: return launch_router<bf16_t>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+        default: return launch_router<f16_t>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+    }
+}

@@ -1,0 +1,100 @@
+"""``FlashMoE`` block on the HIP forward path.
+
+Drop-in for ``flash_moe.modules.flash_moe`` of flash-algo/flash-moe: ``FlashMoEConfig`` takes the same
+six arguments (flash_moe/modules/flash_moe.py:12-27), ``FlashMoE`` owns parameters and buffers under
+the same ``state_dict`` names (:43-53) and ``forward`` returns the same ``(hidden_states, router_logits)``
+pair (:55-105).
+
+Stages of ``forward`` and where each runs:
+  batch-norm + router gate     torch (statistics and a [T,H]x[H,2nk] product)
+  log-softmax                  torch, always in fp32
+  product-key top-k + gates    ``fmoe_router_topk``   (HIP)
+  routed experts               ``fmoe_expert_forward`` (HIP)
+  shared SwiGLU MLP + add      ``fmoe_mlp_forward``    (HIP; the add is the second GEMM's epilogue)
+
+Routing is evaluated in fp32 whatever the module dtype: the normalised activations are rounded to the
+module dtype exactly as the reference does, but their product with the router gate, the log-softmax
+and the pair sums stay in fp32.  With 16-bit log-probabilities the pair sums of the reference are
+tie-dominated (values near -10 are 2^-4 apart in bf16) and which of the tied experts it picks is not
+defined; fp32 scores make the selection well defined.  The returned ``router_logits`` are rounded to
+the module dtype as in the reference.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from flash_moe.ops.hip.flash_expert import expert_forward
+from flash_moe.ops.hip.flash_mlp import mlp_forward
+from flash_moe.ops.hip.flash_router import router_topk_gates
+
+_SILU_NAMES = ("silu", "swish")
+
+
+class FlashMoEConfig:
+    """Plain configuration record; argument order and names as in the reference."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, hidden_act: str, num_experts: int,
+                 num_experts_per_tok: int, norm_topk_prob: bool = False):
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.hidden_act = hidden_act
+        self.num_experts = num_experts
+        self.num_experts_per_tok = num_experts_per_tok
+        self.norm_topk_prob = norm_topk_prob
+
+    def __repr__(self) -> str:
+        body = ", ".join(f"{k}={v!r}" for k, v in vars(self).items())
+        return f"FlashMoEConfig({body})"
+
+
+class FlashMoE(nn.Module):
+    def __init__(self, config: FlashMoEConfig):
+        super().__init__()
+        if config.hidden_act not in _SILU_NAMES:
+            # the fused kernels hard-code SiLU, as the reference's do (flash_expert.py:8-10, flash_mlp.py:8-10)
+            raise ValueError(f"hidden_act={config.hidden_act!r}: the HIP kernels implement 'silu' only")
+        H, I, E = config.hidden_size, config.intermediate_size, config.num_experts
+        self.hidden_size, self.intermediate_size, self.num_experts = H, I, E
+        self.act_fn = F.silu
+        # experts are addressed by a pair of sub-keys; ids >= num_keys**2 are never selected (:38)
+        self.num_keys = math.floor(math.sqrt(E))
+        self.top_k = config.num_experts_per_tok
+        self.norm_topk_prob = config.norm_topk_prob
+
+        self.gate_proj = nn.Linear(H, I, bias=False)
+        self.up_proj = nn.Linear(H, I, bias=False)
+        self.down_proj = nn.Linear(I, H, bias=False)
+
+        self.router_gate = nn.Linear(H, 2 * self.num_keys, bias=False)
+        self.router_norm = nn.BatchNorm1d(H, affine=False)
+
+        self.down_embed = nn.Embedding(E, H)
+        self.up_embed = nn.Embedding(E, H)
+
+    def route(self, tokens: torch.Tensor):
+        """[T, H] -> (router_logits [2, T, nk] in the module dtype, scores, indices int64, gates)."""
+        T = tokens.shape[0]
+        q = self.router_norm(tokens)
+        logits32 = F.linear(q.float(), self.router_gate.weight.float())          # [T, 2*nk], fp32
+        log_probs = F.log_softmax(logits32.view(T, 2, self.num_keys), dim=-1).transpose(0, 1)
+        scores, indices, gates = router_topk_gates(
+            log_probs, self.num_keys, self.top_k, with_gates=True, norm_topk_prob=self.norm_topk_prob
+        )
+        router_logits = logits32.to(tokens.dtype).view(T, 2, self.num_keys).transpose(0, 1)
+        return router_logits, scores, indices, gates
+
+    def forward(self, hidden_states: torch.Tensor, **kwargs):
+        bsz, seq_len, _ = hidden_states.shape
+        tokens = hidden_states.view(-1, self.hidden_size)
+        router_logits, _, indices, gates = self.route(tokens)
+        experts_states = expert_forward(
+            tokens, self.down_embed.weight, self.up_embed.weight, indices, gates.to(tokens.dtype)
+        )
+        out = mlp_forward(
+            tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, residual=experts_states
+        )
+        return out.view(bsz, seq_len, -1), router_logits

@@ -1,0 +1,61 @@
+"""Routed-expert op: ``out[t] = sum_k silu(<x_t, Wd[idx[t,k]]>) * g[t,k] * Wu[idx[t,k]]``.
+
+Same call signature and return value as ``triton_flash_expert_func``
+(flash_moe/ops/triton/flash_expert.py:831-836; contract docs/flash_expert.md:17-58); the work is done
+by ``fmoe_expert_forward`` in libflashmoe_hip.so.
+"""
+from __future__ import annotations
+
+import torch
+
+from flash_moe import _C
+from flash_moe.ops.utils import ensure_contiguous
+
+
+def expert_forward(hidden_states, down_weights, up_weights, indices, routing_weights) -> torch.Tensor:
+    if hidden_states.dim() != 2 or down_weights.dim() != 2 or up_weights.dim() != 2:
+        raise ValueError("hidden_states, down_weights and up_weights must be 2-D")
+    if indices.dim() != 2 or routing_weights.shape != indices.shape:
+        raise ValueError("indices and routing_weights must both be (num_tokens, num_experts_per_tok)")
+    num_tokens, hidden = hidden_states.shape
+    num_experts = down_weights.shape[0]
+    if down_weights.shape != (num_experts, hidden) or up_weights.shape != (num_experts, hidden):
+        raise ValueError("down_weights and up_weights must be (num_experts, hidden_size)")
+    if indices.shape[0] != num_tokens:
+        raise ValueError("indices has a different number of tokens than hidden_states")
+    if indices.dtype != torch.int64:
+        raise TypeError(f"indices must be int64 (got {indices.dtype})")
+    dtype = hidden_states.dtype
+    for name, t in (("down_weights", down_weights), ("up_weights", up_weights), ("routing_weights", routing_weights)):
+        if t.dtype != dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, hidden_states has {dtype}")
+    dev = _C.require_gpu(hidden_states, down_weights, up_weights, indices, routing_weights)
+    x, wd, wu, idx, g = (t.contiguous() for t in (hidden_states, down_weights, up_weights, indices, routing_weights))
+    top_k = idx.shape[1]
+    code = _C.dtype_code(dtype)
+    out = torch.empty_like(x)
+    L = _C.lib()
+    ws_bytes = L.fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, code)
+    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8) if ws_bytes else None
+    with torch.cuda.device(dev):
+        status = L.fmoe_expert_forward(
+            _C.ptr(x), _C.ptr(wd), _C.ptr(wu), _C.ptr(idx), _C.ptr(g), num_tokens, hidden, num_experts, top_k,
+            code, _C.ptr(out), _C.ptr(ws), ws_bytes, _C.current_stream(dev),
+        )
+    _C.check(status, "flash_expert")
+    return out
+
+
+class FlashExpertFunc(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, hidden_states, down_weights, up_weights, indices, routing_weights):
+        return expert_forward(hidden_states, down_weights, up_weights, indices, routing_weights)
+
+    @staticmethod
+    def backward(ctx, dexperts_states):
+        raise NotImplementedError("flash_expert backward is not implemented in the HIP path (forward only)")
+
+
+def flash_expert_func(hidden_states, down_weights, up_weights, indices, routing_weights):
+    return FlashExpertFunc.apply(hidden_states, down_weights, up_weights, indices, routing_weights)

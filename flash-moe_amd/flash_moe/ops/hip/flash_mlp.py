@@ -1,0 +1,63 @@
+"""Shared SwiGLU MLP op: ``(silu(x Wg^T) * (x Wu^T)) Wd^T``.
+
+Same call signature and return value as ``triton_flash_mlp_func``
+(flash_moe/ops/triton/flash_mlp.py:169-181); the work is done by ``fmoe_mlp_forward`` in
+libflashmoe_hip.so (two MFMA GEMMs, the activation fused into the first one's epilogue).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from flash_moe import _C
+from flash_moe.ops.utils import ensure_contiguous
+
+
+def mlp_forward(x, gate_weight, up_weight, down_weight, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x`` may have any leading shape; the last dimension is the hidden size.  ``residual`` (same shape
+    as the output) is added in the second GEMM's epilogue (the add of flash_moe/modules/flash_moe.py:101)."""
+    hidden = x.shape[-1]
+    inter = gate_weight.shape[0]
+    if gate_weight.shape != (inter, hidden) or up_weight.shape != (inter, hidden) or down_weight.shape != (hidden, inter):
+        raise ValueError("expected gate_weight/up_weight (intermediate, hidden) and down_weight (hidden, intermediate)")
+    dtype = x.dtype
+    for name, t in (("gate_weight", gate_weight), ("up_weight", up_weight), ("down_weight", down_weight)):
+        if t.dtype != dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, x has {dtype}")
+    dev = _C.require_gpu(x, gate_weight, up_weight, down_weight, residual)
+    x2 = x.contiguous().view(-1, hidden)
+    num_tokens = x2.shape[0]
+    res = None
+    if residual is not None:
+        if residual.shape != x.shape or residual.dtype != dtype:
+            raise ValueError("residual must have the shape and dtype of x")
+        res = residual.contiguous().view(-1, hidden)
+    wg, wu, wd = gate_weight.contiguous(), up_weight.contiguous(), down_weight.contiguous()
+    code = _C.dtype_code(dtype)
+    out = torch.empty_like(x2)
+    L = _C.lib()
+    ws_bytes = L.fmoe_mlp_workspace_bytes(num_tokens, hidden, inter, code)
+    ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        status = L.fmoe_mlp_forward(
+            _C.ptr(x2), _C.ptr(wg), _C.ptr(wu), _C.ptr(wd), num_tokens, hidden, inter, code, _C.ptr(res),
+            _C.ptr(out), _C.ptr(ws), ws_bytes, _C.current_stream(dev),
+        )
+    _C.check(status, "flash_mlp")
+    return out.view(x.shape)
+
+
+class FlashMLPFunc(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, x, gate_weight, up_weight, down_weight):
+        return mlp_forward(x, gate_weight, up_weight, down_weight)
+
+    @staticmethod
+    def backward(ctx, dout):
+        raise NotImplementedError("flash_mlp backward is not implemented in the HIP path (forward only)")
+
+
+def flash_mlp_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor, down_weight: torch.Tensor) -> torch.Tensor:
+    return FlashMLPFunc.apply(x, gate_weight, up_weight, down_weight)

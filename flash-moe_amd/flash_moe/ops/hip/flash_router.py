@@ -1,0 +1,72 @@
+"""Product-key router op: top-k over the nk*nk pair sums of two per-token score vectors.
+
+Same call signature, return values and argument checks as ``triton_flash_router_func``
+(flash_moe/ops/triton/flash_router.py:381-382; contract docs/flash_router.md:16-40); the work is done
+by ``fmoe_router_topk`` in libflashmoe_hip.so.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from flash_moe import _C
+from flash_moe.ops.utils import ensure_contiguous
+
+
+def router_topk_gates(
+    router_logits: torch.Tensor,
+    num_expert_keys: int,
+    num_experts_per_tok: int,
+    with_gates: bool = False,
+    norm_topk_prob: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Launch the router kernel.  Returns ``(scores, indices, gates-or-None)``.
+
+    ``gates = exp(scores)`` (divided by its per-token sum if ``norm_topk_prob``) is what
+    FlashMoE.forward computes right after the router (flash_moe/modules/flash_moe.py:80-85); asking
+    for it here saves two or three elementwise launches.
+    """
+    # the three checks of _flash_router_forward (flash_router.py:257-263), same exception type
+    assert router_logits.dim() == 3, (
+        "router_logits must be a 3D tensor of shape (2, batch_size * seq_len, num_expert_keys)"
+    )
+    assert router_logits.size(0) == 2, "The first dimension of router_logits must be 2"
+    assert 0 <= num_experts_per_tok <= num_expert_keys, (
+        f"num_experts_per_tok should be in [0, {num_expert_keys}], but got {num_experts_per_tok}"
+    )
+    if router_logits.size(2) != num_expert_keys:
+        raise ValueError(
+            f"router_logits.size(-1)={router_logits.size(2)} does not match num_expert_keys={num_expert_keys}"
+        )
+    dev = _C.require_gpu(router_logits)
+    lp = router_logits.contiguous()
+    num_tokens = lp.size(1)
+    scores = torch.empty((num_tokens, num_experts_per_tok), device=dev, dtype=lp.dtype)
+    indices = torch.empty((num_tokens, num_experts_per_tok), device=dev, dtype=torch.int64)
+    gates = torch.empty_like(scores) if with_gates else None
+    with torch.cuda.device(dev):
+        status = _C.lib().fmoe_router_topk(
+            _C.ptr(lp), num_tokens, num_expert_keys, num_experts_per_tok, _C.dtype_code(lp.dtype),
+            _C.ptr(scores), _C.ptr(indices), _C.ptr(gates), int(bool(norm_topk_prob)), _C.current_stream(dev),
+        )
+    _C.check(status, "flash_router")
+    return scores, indices, gates
+
+
+class FlashRouterFunc(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, router_logits, num_expert_keys, num_experts_per_tok):
+        """router_logits [2, T, nk] -> scores [T, K] (dtype of the input), indices [T, K] int64."""
+        scores, indices, _ = router_topk_gates(router_logits, num_expert_keys, num_experts_per_tok)
+        ctx.mark_non_differentiable(indices)
+        return scores, indices
+
+    @staticmethod
+    def backward(ctx, dscores, dindices):
+        raise NotImplementedError("flash_router backward is not implemented in the HIP path (forward only)")
+
+
+def flash_router_func(router_logits, num_expert_keys, num_experts_per_tok):
+    return FlashRouterFunc.apply(router_logits, num_expert_keys, num_experts_per_tok)

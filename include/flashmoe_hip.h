@@ -1,0 +1,109 @@
+/*
+ * flashmoe_hip.h -- C ABI of the MI355X (gfx950) FlashMoE forward path.
+ *
+ * The reference (flash-algo/flash-moe) has no C ABI: its hot path is three Python entry points
+ * that launch Triton kernels on the caller's current stream.  Each function below is what a
+ * binding for one of those entry points calls instead; the comment on each names the reference
+ * interface it replaces.  All tensors are dense row-major device buffers owned by the caller
+ * (torch); the library never allocates or frees device memory, never synchronises the host, and
+ * launches only on the stream it is given (a hipStream_t passed as void*; NULL = default stream).
+ *
+ * Return value: 0 on success, a negative fmoe_status_t for a rejected argument, or a positive
+ * hipError_t if a launch failed.  fmoe_last_error() returns a thread-local description.
+ */
+#ifndef FLASHMOE_HIP_H
+#define FLASHMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMOE_ABI_VERSION 1
+
+/* element type of activations / weights / scores */
+typedef enum {
+    FMOE_F32 = 0,
+    FMOE_BF16 = 1,
+    FMOE_F16 = 2
+} fmoe_dtype_t;
+
+typedef enum {
+    FMOE_OK = 0,
+    FMOE_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+    FMOE_ERR_BAD_SHAPE = -2,      /* negative / zero / inconsistent extent */
+    FMOE_ERR_TOPK_RANGE = -3,     /* top_k outside [0, num_keys]            (flash_router.py:261-263) */
+    FMOE_ERR_BAD_DTYPE = -4,      /* dtype not one of fmoe_dtype_t */
+    FMOE_ERR_UNSUPPORTED = -5,    /* extent beyond what the kernels are built for (message says which) */
+    FMOE_ERR_ALIGNMENT = -6,      /* pointer not 16-byte aligned or row length not a multiple of 16 bytes */
+    FMOE_ERR_WORKSPACE = -7       /* workspace NULL or smaller than the *_workspace_bytes() figure */
+} fmoe_status_t;
+
+/* ABI version of the loaded library (== FMOE_ABI_VERSION it was built with). */
+int fmoe_abi_version(void);
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char* fmoe_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Product-key router.
+ * Replaces triton_flash_router_func / FlashRouterFunc.forward / _flash_router_forward
+ * (flash_moe/ops/triton/flash_router.py:381-382, 347-368, 252-314; contract docs/flash_router.md:16-40),
+ * and, when `gates` is given, the two statements after it in FlashMoE.forward
+ * (flash_moe/modules/flash_moe.py:80-85: exp, optional renormalisation).
+ *
+ *   log_probs  [2, num_tokens, num_keys]  dtype      per-half scores (log-probabilities in the module)
+ *   scores     [num_tokens, top_k]        dtype      K largest sums lp[0,t,i]+lp[1,t,j], descending;
+ *                                                    16-bit dtypes: each sum rounded to dtype, as the
+ *                                                    reference adds in the input dtype (flash_router.py:51-53)
+ *   indices    [num_tokens, top_k]        int64      i*num_keys + j; ties to the lower index (tl.argmax rule)
+ *   gates      [num_tokens, top_k]        dtype      optional (NULL to skip): exp(score), divided by the
+ *                                                    per-token sum when norm_topk_prob != 0
+ * Requires 0 <= top_k <= num_keys (same rule as the reference's assert), num_keys <= 1024, top_k <= 256.
+ */
+int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
+                     void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Routed experts.
+ * Replaces triton_flash_expert_func / FlashExpertFunc.forward / _flash_expert_forward and its host-side
+ * preprocessing (flash_moe/ops/triton/flash_expert.py:831-836, 748-796, 580-651, 528-577; contract
+ * docs/flash_expert.md:17-58):
+ *   out[t,:] = sum_k silu(<x[t,:], down[idx[t,k],:]>) * gates[t,k] * up[idx[t,k],:]
+ *
+ *   x [T,H], down [E,H], up [E,H], gates [T,K], out [T,H]: dtype;  indices [T,K]: int64 in [0,E).
+ * Duplicate ids in a row add, as in the reference.  An id outside [0,E) contributes nothing (the
+ * reference reads out of bounds).  Accumulation is fp32 and deterministic (no atomics); `out` is
+ * written once, it need not be zeroed.
+ * fmoe_expert_workspace_bytes() gives the scratch the call needs (may be 0); pass a 256-byte aligned
+ * buffer of at least that size.
+ */
+size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
+
+int fmoe_expert_forward(const void* x, const void* down, const void* up, const int64_t* indices,
+                        const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k,
+                        int dtype, void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Shared SwiGLU MLP.
+ * Replaces triton_flash_mlp_func / TritonSwiGLUFunc.forward / swiglu_forward
+ * (flash_moe/ops/triton/flash_mlp.py:169-181, 153-159, 105-123) and, when `residual` is given, the add
+ * that follows it in FlashMoE.forward (flash_moe/modules/flash_moe.py:101):
+ *   out = (silu(x gate_w^T) * (x up_w^T)) down_w^T  [+ residual]
+ *
+ *   x [T,H], gate_w [I,H], up_w [I,H], down_w [H,I], residual [T,H] or NULL, out [T,H]: dtype.
+ * The gate/up products are kept in fp32 until after silu(.)*(.), then rounded once to dtype.
+ * workspace: fmoe_mlp_workspace_bytes() bytes (the [T,I] activation), 256-byte aligned.
+ */
+size_t fmoe_mlp_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int dtype);
+
+int fmoe_mlp_forward(const void* x, const void* gate_w, const void* up_w, const void* down_w,
+                     int64_t num_tokens, int hidden, int intermediate, int dtype, const void* residual,
+                     void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHMOE_HIP_H */

@@ -1,0 +1,105 @@
+"""The C-ABI library: loads without a GPU, exports every symbol the header declares, and rejects bad
+arguments with the documented status codes before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from flash_moe import _C
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flashmoe_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmoe_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("fmoe_router_topk", "fmoe_expert_forward", "fmoe_mlp_forward", "fmoe_last_error", "fmoe_abi_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _C.lib()
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} declared in flashmoe_hip.h but not exported by {_C.lib_path()}"
+    # and the Python binding table names exactly the declared functions
+    assert sorted(_C.SIGNATURES) == declared_functions()
+    assert lib.fmoe_abi_version() == _C.ABI_VERSION
+
+
+def test_citations_in_header_point_at_the_reference_interface():
+    text = open(HEADER).read()
+    for cite in ("flash_router.py:381-382", "flash_expert.py:831-836", "flash_mlp.py:169-181", "flash_moe.py:101"):
+        assert cite in text
+
+
+def _buf(n=4096):
+    b = ctypes.create_string_buffer(n + 256)
+    addr = (ctypes.addressof(b) + 255) // 256 * 256
+    return b, addr
+
+
+def test_router_argument_checks():
+    lib = _C.lib()
+    keep, a = _buf()
+    # top_k outside [0, nk]: the reference's assertion (flash_router.py:261-263)
+    assert lib.fmoe_router_topk(a, 4, 8, 9, _C.F32, a, a, None, 0, None) == -3
+    assert b"[0, 8]" in lib.fmoe_last_error()
+    assert lib.fmoe_router_topk(a, 4, 8, -1, _C.F32, a, a, None, 0, None) == -3
+    assert lib.fmoe_router_topk(a, 4, 8, 4, 7, a, a, None, 0, None) == -4          # dtype
+    assert lib.fmoe_router_topk(a, -1, 8, 4, _C.F32, a, a, None, 0, None) == -2     # shape
+    assert lib.fmoe_router_topk(None, 4, 8, 4, _C.F32, a, a, None, 0, None) == -1   # null
+    assert lib.fmoe_router_topk(a, 4, 512, 300, _C.F32, a, a, None, 0, None) == -5  # top_k > 256
+    # empty problems succeed without a launch
+    assert lib.fmoe_router_topk(None, 0, 8, 4, _C.F32, None, None, None, 0, None) == 0
+    assert lib.fmoe_router_topk(a, 4, 8, 0, _C.F32, a, a, None, 0, None) == 0
+    assert lib.fmoe_last_error() == b""
+
+
+def test_expert_argument_checks():
+    lib = _C.lib()
+    keep, a = _buf()
+    f = lib.fmoe_expert_forward
+    assert f(a, a, a, a, a, 4, 64, 16, 2, 9, a, None, 0, None) == -4
+    assert f(a, a, a, a, a, 4, 0, 16, 2, _C.BF16, a, None, 0, None) == -2
+    assert f(None, a, a, a, a, 4, 64, 16, 2, _C.BF16, a, None, 0, None) == -1
+    assert f(a, a, a, None, a, 4, 64, 16, 2, _C.BF16, a, None, 0, None) == -1
+    assert f(a, a, a, a, a, 4, 60, 16, 2, _C.BF16, a, None, 0, None) == -6          # row not 16-byte multiple
+    assert f(a + 2, a, a, a, a, 4, 64, 16, 2, _C.BF16, a, None, 0, None) == -6      # misaligned pointer
+    assert f(a, a, a, a, a, 4, 1 << 20, 16, 2, _C.BF16, a, None, 0, None) == -5      # hidden too large
+    assert f(None, None, None, None, None, 0, 64, 16, 2, _C.BF16, None, None, 0, None) == 0
+    assert isinstance(lib.fmoe_expert_workspace_bytes(1024, 1024, 16384, 64, _C.BF16), int)
+
+
+def test_mlp_argument_checks():
+    lib = _C.lib()
+    keep, a = _buf()
+    f = lib.fmoe_mlp_forward
+    need = lib.fmoe_mlp_workspace_bytes(8, 64, 128, _C.BF16)
+    assert need >= 8 * 128 * 2 and need % 256 == 0
+    assert lib.fmoe_mlp_workspace_bytes(8, 64, 128, _C.F32) >= 8 * 128 * 4
+    assert f(a, a, a, a, 8, 64, 128, 5, None, a, a, need, None) == -4
+    assert f(a, a, a, a, 8, 64, -1, _C.BF16, None, a, a, need, None) == -2
+    assert f(a, None, a, a, 8, 64, 128, _C.BF16, None, a, a, need, None) == -1
+    assert f(a, a, a, a, 8, 64, 128, _C.BF16, None, a, a, need - 1, None) == -7
+    assert f(a, a, a, a, 8, 64, 128, _C.BF16, None, a, None, need, None) == -7
+    assert f(a, a, a, a, 8, 60, 128, _C.BF16, None, a, a, need, None) == -6
+    assert f(None, None, None, None, 0, 64, 128, _C.BF16, None, None, None, 0, None) == 0
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    from flash_moe.ops import flash_expert_func, flash_mlp_func, flash_router_func
+
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        flash_router_func(torch.zeros(2, 4, 8), 8, 2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        flash_expert_func(torch.zeros(4, 8), torch.zeros(16, 8), torch.zeros(16, 8), torch.zeros(4, 2, dtype=torch.int64), torch.zeros(4, 2))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        flash_mlp_func(torch.zeros(4, 8), torch.zeros(16, 8), torch.zeros(16, 8), torch.zeros(8, 16))

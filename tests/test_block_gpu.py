@@ -1,0 +1,108 @@
+"""Whole-block parity: FlashMoE (HIP path) against the CPU oracle of FlashMoE_Pytorch.forward."""
+import pytest
+import torch
+
+from helpers import assert_output_close, cuda, rel_fro
+from oracle import flashmoe_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def build(H, I, E, K, norm, dtype, seed=0, std=0.02):
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+
+    w = orc.make_block_weights(H, I, E, seed=seed, std=std).to(dtype)
+    m = FlashMoE(FlashMoEConfig(H, I, "silu", E, K, norm))
+    m.load_state_dict({"gate_proj.weight": w.gate_proj, "up_proj.weight": w.up_proj, "down_proj.weight": w.down_proj,
+                       "router_gate.weight": w.router_gate, "down_embed.weight": w.down_embed,
+                       "up_embed.weight": w.up_embed}, strict=False)
+    return m.to(device="cuda", dtype=dtype), w
+
+
+def stagewise_check(m, w, x, K, norm, dtype):
+    """End-to-end comparison plus a stage-by-stage one that feeds the oracle the HIP path's own
+    intermediates, so that one flipped near-tie in the router cannot hide or fake an error downstream."""
+    H = x.shape[-1]
+    T = x.shape[0] * x.shape[1]
+    nk = w.num_keys
+    y, logits = m(x.cuda())
+    assert y.shape == x.shape and y.dtype == dtype and logits.shape == (2, T, nk) and logits.dtype == dtype
+    w.running_mean.zero_(); w.running_var.fill_(1.0)
+    ref = orc.block_forward(x, w, K, norm_topk_prob=norm, training=True, routing_fp32=True, token_chunk=256)
+    assert_output_close(logits, ref["router_logits"], dtype, "router_logits")
+    assert_output_close(y, ref["y"], dtype, "block output")
+    # running statistics follow nn.BatchNorm1d
+    torch.testing.assert_close(m.router_norm.running_mean.float().cpu(), w.running_mean.float(), rtol=2e-2, atol=1e-3)
+    torch.testing.assert_close(m.router_norm.running_var.float().cpu(), w.running_var.float(), rtol=2e-2, atol=1e-3)
+
+    # stage by stage on the HIP path's intermediates
+    m.router_norm.reset_running_stats()
+    tokens = x.cuda().view(-1, H)
+    _, scores, indices, gates = m.route(tokens)
+    idx_cpu, gates_cpu = indices.cpu(), gates.cpu()
+    # router: share of tokens whose expert set is the oracle's (a near-tie may flip on a different fp32 summation order)
+    same = (idx_cpu.sort(-1).values == ref["indices"].sort(-1).values).all(-1).float().mean().item()
+    assert same > 0.9, f"only {same:.3f} of the tokens select the oracle's expert set"
+    # experts: oracle on the HIP path's own indices and gates
+    from flash_moe.ops.hip.flash_expert import expert_forward
+
+    e_hip = expert_forward(tokens, m.down_embed.weight, m.up_embed.weight, indices, gates.to(dtype)).cpu()
+    e_ref = orc.expert_forward(x.view(-1, H).double(), w.down_embed.double(), w.up_embed.double(), idx_cpu,
+                               gates_cpu.to(dtype).double(), token_chunk=256)
+    fro = rel_fro(e_hip, e_ref)
+    assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 1e-3}[dtype], f"experts: {fro:.3e}"
+    return same
+
+
+@pytest.mark.parametrize("norm", [False, True])
+def test_block_c1_fp32(norm):
+    # C1: fp32, 1 x 512 tokens, H=256, I=1024, E=1024 (32x32 keys), K=16
+    m, w = build(256, 1024, 1024, 16, norm, torch.float32)
+    x = torch.randn(1, 512, 256, generator=torch.Generator().manual_seed(0))
+    same = stagewise_check(m, w, x, 16, norm, torch.float32)
+    assert same > 0.97
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_block_c4_shape_fewer_tokens(dtype):
+    # C4 weights (H=1024, I=4096, E=16384, K=64) on 512 tokens so that the CPU oracle finishes in seconds
+    m, w = build(1024, 4096, 16384, 64, False, dtype)
+    x = torch.randn(1, 512, 1024, generator=torch.Generator().manual_seed(0)).to(dtype)
+    stagewise_check(m, w, x, 64, False, dtype)
+
+
+def test_block_c4_full_size_properties():
+    # C4 at full size (README configuration): structure and size-independent properties
+    dtype = torch.bfloat16
+    m, w = build(1024, 4096, 16384, 64, False, dtype)
+    x = torch.randn(1, 4096, 1024, generator=torch.Generator().manual_seed(0)).to(dtype).cuda()
+    y, logits = m(x)
+    assert y.shape == (1, 4096, 1024) and logits.shape == (2, 4096, 128)
+    assert torch.isfinite(y).all() and torch.isfinite(logits).all()
+    m.eval()
+    y1, _ = m(x)
+    y2, _ = m(x)
+    assert torch.equal(y1, y2)                               # deterministic
+    # in eval mode tokens are independent: a slice of the batch gives the same rows
+    ys, _ = m(x[:, 1000:1512])
+    assert rel_fro(ys, y1[:, 1000:1512]) < 1e-3
+    # block = shared MLP + routed experts
+    from flash_moe.ops import flash_mlp_func
+    from flash_moe.ops.hip.flash_expert import expert_forward
+
+    tokens = x.view(-1, 1024)
+    _, _, indices, gates = m.route(tokens)
+    parts = flash_mlp_func(tokens, m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight).float() + expert_forward(
+        tokens, m.down_embed.weight, m.up_embed.weight, indices, gates.to(dtype)).float()
+    assert rel_fro(y1.view(-1, 1024), parts) < 6e-3
+    # gates are probabilities p_x * p_y of distinct experts
+    assert (gates > 0).all() and (gates.sum(-1) <= 1 + 1e-3).all()
+    assert (indices.sort(-1).values.diff(dim=-1) != 0).all() and indices.max() < 16384
+
+
+def test_block_c5_shape_fewer_tokens():
+    # C5 weights scaled to fit a quick run: H=2048, I=8192, 512x512 keys, K=128, normalised gates, 256 tokens
+    dtype = torch.bfloat16
+    m, w = build(2048, 8192, 262144, 128, True, dtype)
+    x = torch.randn(1, 256, 2048, generator=torch.Generator().manual_seed(0)).to(dtype)
+    stagewise_check(m, w, x, 128, True, dtype)

@@ -1,0 +1,115 @@
+"""Parity of the HIP routed-expert op with the CPU oracle, through the op (and so the C ABI)."""
+import pytest
+import torch
+
+from helpers import assert_output_close, cuda, rel_fro
+from oracle import flashmoe_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def run(x, wd, wu, idx, g):
+    from flash_moe.ops import flash_expert_func
+
+    return flash_expert_func(*cuda(x, wd, wu, idx, g)).cpu()
+
+
+def truth64(x, wd, wu, idx, g):
+    """The oracle evaluated in float64 on the (already rounded) inputs."""
+    return orc.expert_forward(x.double(), wd.double(), wu.double(), idx, g.double())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,K", [
+    (512, 256, 1024, 16),        # C1
+    (1024, 1024, 16384, 64),     # C3 / C4 row shape, fewer tokens
+    (256, 2048, 4096, 128),      # C5 row shape
+    (37, 72, 50, 5),             # ragged: rows of 9 packets, token count not a multiple of the block
+    (3, 8, 4, 1),
+])
+def test_expert_matches_oracle(dtype, T, H, E, K):
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=T + K)
+    x, wd, wu, g = (t.to(dtype) for t in (x, wd, wu, g))
+    got = run(x, wd, wu, idx, g)
+    assert got.dtype == dtype and got.shape == (T, H)
+    # (1) the stated bar: against the oracle run in the same dtype
+    assert_output_close(got, orc.expert_forward(x, wd, wu, idx, g), dtype, "expert vs oracle")
+    # (2) against the float64 evaluation of the same rounded inputs: only the final rounding remains
+    fro = rel_fro(got, truth64(x, wd, wu, idx, g))
+    assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 5e-4}[dtype], fro
+
+
+def test_expert_reference_test_distribution():
+    # distributions of the reference's expert benchmark (tests/test_expert.py:160-175): x ~ N(0,0.5),
+    # tables ~ N(0,0.1), ids drawn WITH replacement, gates ~ N(0,0.1) (negative values allowed)
+    g0 = torch.Generator().manual_seed(0)
+    T, H, E, K = 256, 1024, 4096, 512
+    x = (torch.randn(T, H, generator=g0) * 0.5).bfloat16()
+    wd = (torch.randn(E, H, generator=g0) * 0.1).bfloat16()
+    wu = (torch.randn(E, H, generator=g0) * 0.1).bfloat16()
+    idx = torch.randint(0, E, (T, K), generator=g0)
+    g = (torch.randn(T, K, generator=g0) * 0.1).bfloat16()
+    got = run(x, wd, wu, idx, g)
+    assert rel_fro(got, truth64(x, wd, wu, idx, g)) < 4e-3
+
+
+def test_expert_properties_full_size():
+    # C3 at full size: size-independent properties instead of a CPU evaluation of all 1M pairs
+    T, H, E, K = 16384, 1024, 16384, 64
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=0)
+    x, wd, wu, g = (t.bfloat16() for t in (x, wd, wu, g))
+    xc, wdc, wuc, idxc, gc = cuda(x, wd, wu, idx, g)
+    from flash_moe.ops import flash_expert_func
+
+    out = flash_expert_func(xc, wdc, wuc, idxc, gc)
+    assert torch.isfinite(out).all()
+    # deterministic: no atomics, so a second run is bit-identical
+    assert torch.equal(out, flash_expert_func(xc, wdc, wuc, idxc, gc))
+    # zero gates -> exact zeros (also proves the output is written, not accumulated into)
+    assert flash_expert_func(xc, wdc, wuc, idxc, torch.zeros_like(gc)).abs().max() == 0
+    # linear in the gates (power-of-two factor: exact in bf16)
+    assert torch.equal(flash_expert_func(xc, wdc, wuc, idxc, gc * 2), out * 2)
+    # permuting the K slots of every token only changes the fp32 summation order
+    perm = torch.randperm(K, generator=torch.Generator().manual_seed(1)).cuda()
+    out_p = flash_expert_func(xc, wdc, wuc, idxc[:, perm].contiguous(), gc[:, perm].contiguous())
+    assert rel_fro(out_p, out) < 4e-3
+    # a slice of tokens against the oracle
+    sl = slice(5000, 5512)
+    assert_output_close(out[sl].cpu(), orc.expert_forward(x[sl], wd, wu, idx[sl], g[sl]), torch.bfloat16, "C3 slice")
+    assert rel_fro(out[sl].cpu(), truth64(x[sl], wd, wu, idx[sl], g[sl])) < 4e-3
+
+
+def test_expert_duplicates_and_single_expert():
+    T, H, E = 64, 256, 32
+    x, wd, wu, _, _ = orc.make_expert_inputs(T, H, E, 4, seed=5, std=0.2)
+    e = torch.full((T, 4), 7, dtype=torch.int64)
+    one = run(x, wd, wu, e[:, :1].contiguous(), torch.ones(T, 1))
+    rep = run(x, wd, wu, e, torch.full((T, 4), 0.25))
+    torch.testing.assert_close(rep, one, rtol=1e-5, atol=1e-7)
+    s = x @ wd[7]
+    torch.testing.assert_close(one, (torch.nn.functional.silu(s)).unsqueeze(-1) * wu[7], rtol=1e-4, atol=1e-6)
+
+
+def test_expert_out_of_range_ids_contribute_nothing():
+    T, H, E, K = 32, 64, 16, 4
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=6, std=0.2)
+    bad = idx.clone()
+    bad[:, 0] = E + 3
+    bad[::2, 1] = -1
+    g2 = g.clone()
+    g2[:, 0] = 0
+    g2[::2, 1] = 0
+    torch.testing.assert_close(run(x, wd, wu, bad, g), run(x, wd, wu, idx, g2), rtol=1e-6, atol=1e-8)
+
+
+def test_expert_empty_and_noncontiguous():
+    from flash_moe.ops import flash_expert_func
+
+    T, H, E, K = 16, 64, 16, 4
+    x, wd, wu, idx, g = cuda(*orc.make_expert_inputs(T, H, E, K, seed=7))
+    assert flash_expert_func(x[:0], wd, wu, idx[:0], g[:0]).shape == (0, H)
+    z = flash_expert_func(x, wd, wu, idx[:, :0], g[:, :0])
+    assert z.shape == (T, H) and z.abs().max() == 0
+    xt = x.t().contiguous().t()
+    assert not xt.is_contiguous()
+    assert torch.equal(flash_expert_func(xt, wd, wu, idx, g), flash_expert_func(x, wd, wu, idx, g))

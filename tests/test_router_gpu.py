@@ -1,0 +1,131 @@
+"""Parity of the HIP product-key router with the CPU oracle, through the op (and so the C ABI)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import cuda
+from oracle import bruteforce as bf
+from oracle import flashmoe_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_topk_chunked(lp, nk, K, chunk=512):
+    s, i = [], []
+    for lo in range(0, lp.shape[1], chunk):
+        a, b = orc.router_topk(lp[:, lo:lo + chunk].contiguous(), nk, K)
+        s.append(a); i.append(b)
+    return torch.cat(s), torch.cat(i)
+
+
+def check_fp32_case(lp, nk, K):
+    from flash_moe.ops import flash_router_func
+
+    T = lp.shape[1]
+    scores, idx = flash_router_func(cuda(lp), nk, K)
+    assert scores.shape == (T, K) and idx.shape == (T, K)
+    assert scores.dtype == torch.float32 and idx.dtype == torch.int64
+    scores, idx = scores.cpu(), idx.cpu()
+    # one extra rank from the oracle tells where the cut is a tie
+    Kx = min(K + 1, nk * nk)
+    o_scores, o_idx = oracle_topk_chunked(lp, nk, Kx)
+    # the K largest sums, bit for bit, in descending order
+    assert torch.equal(scores, o_scores[:, :K])
+    # every index reproduces its score exactly, is in range and distinct within the token
+    again = lp[0].gather(-1, idx // nk) + lp[1].gather(-1, idx % nk)
+    assert torch.equal(again, scores)
+    assert idx.min() >= 0 and idx.max() < nk * nk
+    assert (idx.sort(-1).values.diff(dim=-1) != 0).all()
+    # index sets equal the oracle's except where the K-th and (K+1)-th sums are closer than 1e-6
+    same = (idx.sort(-1).values == o_idx[:, :K].sort(-1).values).all(-1)
+    if Kx > K:
+        tie_at_cut = (o_scores[:, K - 1] - o_scores[:, K]).abs() < 1e-6
+        assert (same | tie_at_cut).all(), f"{(~(same | tie_at_cut)).sum().item()} tokens differ without a tie"
+    else:
+        assert same.all()
+    # where no two of the K+1 best sums tie, the order is the oracle's too
+    strict = (o_scores[:, :-1] - o_scores[:, 1:] > 0).all(-1) if Kx > 1 else torch.ones(T, dtype=torch.bool)
+    assert torch.equal(idx[strict], o_idx[:, :K][strict])
+    return scores, idx
+
+
+@pytest.mark.parametrize("T,nk,K", [
+    (4096, 64, 8), (4096, 128, 16),            # shapes of the reference's router test (tests/test_router.py:78-79)
+    (512, 32, 16),                             # C1
+    (8192, 128, 64),                           # C2
+    (300, 512, 128),                           # C5 keys, few tokens
+    (77, 100, 37), (5, 13, 13), (64, 8, 1), (33, 256, 200), (1, 128, 64), (1030, 64, 64),
+])
+def test_router_fp32_log_probs(T, nk, K):
+    check_fp32_case(orc.make_router_inputs(T, nk, seed=T + nk), nk, K)
+
+
+def test_router_fp32_raw_normals():
+    # the reference's own router benchmark feeds raw normals, not log-probabilities (tests/test_router.py:43-46)
+    check_fp32_case(orc.make_router_inputs(2048, 128, seed=0, log_probs=False), 128, 16)
+
+
+def test_router_matches_exhaustive_scan_with_lowest_index_ties():
+    # quantised scores force many exact ties; the exhaustive C scan breaks them to the lowest flat index,
+    # the rule of the reference kernel (tl.argmax).  Scores must agree exactly; indices may differ only
+    # inside a group of equal sums that straddles the cut.
+    from flash_moe.ops import flash_router_func
+
+    T, nk, K = 200, 32, 16
+    lp = (orc.make_router_inputs(T, nk, seed=3) * 2).round() / 2
+    s, i = flash_router_func(cuda(lp), nk, K)
+    b_s, b_i = bf.router_topk(lp.numpy(), nk, K)
+    assert np.array_equal(s.cpu().numpy(), b_s)
+    i = i.cpu()
+    again = lp[0].gather(-1, i // nk) + lp[1].gather(-1, i % nk)
+    assert torch.equal(again, s.cpu())
+    above_cut = torch.from_numpy(b_s) > torch.from_numpy(b_s[:, -1:])
+    for t in range(T):
+        want = set(b_i[t][above_cut[t].numpy()].tolist())      # strictly better than the K-th sum: forced
+        assert want <= set(i[t].tolist())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_router_16bit_scores(dtype):
+    # sums are rounded to the input dtype as the reference adds in the input dtype (flash_router.py:51-53)
+    from flash_moe.ops import flash_router_func
+
+    T, nk, K = 1024, 128, 64
+    lp = orc.make_router_inputs(T, nk, seed=1).to(dtype)
+    s, i = flash_router_func(cuda(lp), nk, K)
+    assert s.dtype == dtype
+    s, i = s.cpu(), i.cpu()
+    o_s, _ = oracle_topk_chunked(lp, nk, K)
+    assert torch.equal(s, o_s)                                   # same multiset of rounded sums, same order
+    again = lp[0].gather(-1, i // nk) + lp[1].gather(-1, i % nk)
+    assert torch.equal(again, s)
+    assert (i.sort(-1).values.diff(dim=-1) != 0).all()
+
+
+@pytest.mark.parametrize("norm", [False, True])
+def test_router_gates(norm):
+    from flash_moe.ops.hip.flash_router import router_topk_gates
+
+    T, nk, K = 777, 128, 64
+    lp = orc.make_router_inputs(T, nk, seed=2)
+    s, i, g = router_topk_gates(cuda(lp), nk, K, with_gates=True, norm_topk_prob=norm)
+    ref = orc.routing_weights(s.cpu(), norm)
+    torch.testing.assert_close(g.cpu(), ref, rtol=1e-5, atol=1e-9)
+    if norm:
+        torch.testing.assert_close(g.sum(-1).cpu(), torch.ones(T), rtol=1e-5, atol=1e-5)
+
+
+def test_router_noncontiguous_input_and_empty():
+    from flash_moe.ops import flash_router_func
+
+    T, nk, K = 64, 32, 8
+    lp = orc.make_router_inputs(T, nk, seed=4)
+    view = cuda(lp.transpose(0, 1).contiguous()).transpose(0, 1)   # [2,T,nk] view of [T,2,nk], as in the module
+    assert not view.is_contiguous()
+    s, i = flash_router_func(view, nk, K)
+    s2, i2 = flash_router_func(cuda(lp), nk, K)
+    assert torch.equal(s, s2) and torch.equal(i, i2)
+    s0, i0 = flash_router_func(cuda(lp), nk, 0)
+    assert s0.shape == (T, 0) and i0.shape == (T, 0)
+    se, ie = flash_router_func(torch.empty(2, 0, nk, device="cuda"), nk, K)
+    assert se.shape == (0, K)
