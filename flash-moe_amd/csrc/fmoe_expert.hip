@@ -16,8 +16,6 @@ namespace {
 constexpr int kPairsInFlight = 4;   // (down,up) row pairs requested ahead per wave
 constexpr int kWavesPerBlock = 4;
 
-template <typename T> struct Row16 { u32x4_t raw; };
-
 // dot of two 16-byte packets, accumulated into acc
 template <typename T> __device__ inline float dot16(u32x4_t a, u32x4_t b, float acc);
 template <> __device__ inline float dot16<float>(u32x4_t a, u32x4_t b, float acc) {
@@ -27,14 +25,19 @@ template <> __device__ inline float dot16<float>(u32x4_t a, u32x4_t b, float acc
 }
 template <> __device__ inline float dot16<bf16_t>(u32x4_t a, u32x4_t b, float acc) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a[i]), __builtin_bit_cast(bf16x2_t, b[i]), acc, false);
+    for (int i = 0; i < 4; ++i) {
+        // element first into a scalar: bit-casting the subscript expression itself reads element 0
+        const uint32_t ai = a[i], bi = b[i];
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, ai), __builtin_bit_cast(bf16x2_t, bi), acc, false);
+    }
     return acc;
 }
 template <> __device__ inline float dot16<f16_t>(u32x4_t a, u32x4_t b, float acc) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a[i]), __builtin_bit_cast(f16x2_t, b[i]), acc, false);
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t ai = a[i], bi = b[i];
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, ai), __builtin_bit_cast(f16x2_t, bi), acc, false);
+    }
     return acc;
 }
 
@@ -54,7 +57,8 @@ template <> __device__ inline void axpy16<bf16_t>(float s, u32x4_t w, float* acc
 template <> __device__ inline void axpy16<f16_t>(float s, u32x4_t w, float* acc) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        f16x2_t p = __builtin_bit_cast(f16x2_t, w[i]);
+        const uint32_t wi = w[i];
+        f16x2_t p = __builtin_bit_cast(f16x2_t, wi);
         acc[2 * i] = __builtin_fmaf(s, (float)p[0], acc[2 * i]);
         acc[2 * i + 1] = __builtin_fmaf(s, (float)p[1], acc[2 * i + 1]);
     }

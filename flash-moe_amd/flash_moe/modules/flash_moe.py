@@ -75,12 +75,19 @@ class FlashMoE(nn.Module):
         self.down_embed = nn.Embedding(E, H)
         self.up_embed = nn.Embedding(E, H)
 
+    def router_log_probs(self, tokens: torch.Tensor):
+        """[T, H] -> (logits [T, 2*nk] fp32, log-probabilities [2, T, nk] fp32).  In training mode this
+        updates the batch-norm running statistics, like any call of the module."""
+        T = tokens.shape[0]
+        q = self.router_norm(tokens)
+        logits32 = F.linear(q.float(), self.router_gate.weight.float())
+        log_probs = F.log_softmax(logits32.view(T, 2, self.num_keys), dim=-1).transpose(0, 1)
+        return logits32, log_probs
+
     def route(self, tokens: torch.Tensor):
         """[T, H] -> (router_logits [2, T, nk] in the module dtype, scores, indices int64, gates)."""
         T = tokens.shape[0]
-        q = self.router_norm(tokens)
-        logits32 = F.linear(q.float(), self.router_gate.weight.float())          # [T, 2*nk], fp32
-        log_probs = F.log_softmax(logits32.view(T, 2, self.num_keys), dim=-1).transpose(0, 1)
+        logits32, log_probs = self.router_log_probs(tokens)
         scores, indices, gates = router_topk_gates(
             log_probs, self.num_keys, self.top_k, with_gates=True, norm_topk_prob=self.norm_topk_prob
         )

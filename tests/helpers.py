@@ -8,12 +8,12 @@ FRO_TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 2e-3}
 
 
 def rel_fro(a, b):
-    a, b = a.double().cpu(), b.double().cpu()
-    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return float(((a - b).norm() / b.norm().clamp_min(1e-300)).item())
 
 
 def max_rel_to_scale(a, b):
-    a, b = a.double().cpu(), b.double().cpu()
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
     return float((a - b).abs().max() / b.abs().max().clamp_min(1e-300))
 
 
@@ -32,3 +32,16 @@ def assert_output_close(got, ref, dtype, what=""):
 def cuda(*ts):
     out = tuple(None if t is None else t.cuda() for t in ts)
     return out if len(out) > 1 else out[0]
+
+
+def assert_mostly_close(got, ref, dtype, what="", max_outliers=1e-4):
+    """Against an oracle evaluated in a 16-bit dtype: that oracle rounds every intermediate (gate, up,
+    their product, each partial output) to 16 bits, so its own noise reaches the tolerance in the far
+    tail when rows are long.  All but a 1e-4 fraction of the elements must meet rtol = atol, and the
+    scale-aware bounds must hold for the whole tensor."""
+    tol = OUT_TOL[dtype]
+    g, r = got.detach().float().cpu(), ref.detach().float().cpu()
+    bad = ((g - r).abs() > tol + tol * r.abs()).float().mean().item()
+    assert bad <= max_outliers, f"{what}: {bad:.2e} of the elements outside rtol=atol={tol}"
+    assert rel_fro(g, r) <= FRO_TOL[dtype], f"{what}: relative Frobenius error {rel_fro(g, r):.3e}"
+    assert max_rel_to_scale(g, r) <= 2 * tol, f"{what}: max|diff|/max|ref| = {max_rel_to_scale(g, r):.3e}"

@@ -2,7 +2,7 @@
 import pytest
 import torch
 
-from helpers import assert_output_close, cuda, rel_fro
+from helpers import assert_mostly_close, assert_output_close, cuda, rel_fro
 from oracle import flashmoe_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -30,7 +30,10 @@ def stagewise_check(m, w, x, K, norm, dtype):
     w.running_mean.zero_(); w.running_var.fill_(1.0)
     ref = orc.block_forward(x, w, K, norm_topk_prob=norm, training=True, routing_fp32=True, token_chunk=256)
     assert_output_close(logits, ref["router_logits"], dtype, "router_logits")
-    assert_output_close(y, ref["y"], dtype, "block output")
+    if dtype == torch.float32:
+        assert_output_close(y, ref["y"], dtype, "block output")
+    else:
+        assert_mostly_close(y, ref["y"], dtype, "block output vs same-dtype oracle")
     # running statistics follow nn.BatchNorm1d
     torch.testing.assert_close(m.router_norm.running_mean.float().cpu(), w.running_mean.float(), rtol=2e-2, atol=1e-3)
     torch.testing.assert_close(m.router_norm.running_var.float().cpu(), w.running_var.float(), rtol=2e-2, atol=1e-3)
@@ -38,11 +41,25 @@ def stagewise_check(m, w, x, K, norm, dtype):
     # stage by stage on the HIP path's intermediates
     m.router_norm.reset_running_stats()
     tokens = x.cuda().view(-1, H)
+    _, lp = m.router_log_probs(tokens)
+    m.router_norm.reset_running_stats()
     _, scores, indices, gates = m.route(tokens)
     idx_cpu, gates_cpu = indices.cpu(), gates.cpu()
-    # router: share of tokens whose expert set is the oracle's (a near-tie may flip on a different fp32 summation order)
-    same = (idx_cpu.sort(-1).values == ref["indices"].sort(-1).values).all(-1).float().mean().item()
-    assert same > 0.9, f"only {same:.3f} of the tokens select the oracle's expert set"
+    # router stage on identical input: the oracle's top-k of the HIP path's own fp32 log-probabilities
+    lp_cpu = lp.contiguous().cpu()
+    Kx = K + 1
+    o_s = torch.cat([orc.router_topk(lp_cpu[:, lo:lo + 256].contiguous(), nk, Kx)[0] for lo in range(0, T, 256)])
+    o_i = torch.cat([orc.router_topk(lp_cpu[:, lo:lo + 256].contiguous(), nk, Kx)[1] for lo in range(0, T, 256)])
+    assert torch.equal(scores.cpu(), o_s[:, :K])
+    set_equal = (idx_cpu.sort(-1).values == o_i[:, :K].sort(-1).values).all(-1)
+    tie_at_cut = (o_s[:, K - 1] - o_s[:, K]).abs() < 1e-6
+    assert (set_equal | tie_at_cut).all()
+    torch.testing.assert_close(gates_cpu, orc.routing_weights(o_s[:, :K], norm), rtol=1e-5, atol=1e-10)
+    # end to end the selection is chaotic: a one-ulp difference in a 16-bit batch-norm output moves a logit
+    # by ~1e-4 and can swap the experts around the cut, so only the overlap with the oracle's sets is bounded
+    hit = torch.tensor([len(set(a.tolist()) & set(b.tolist())) for a, b in zip(idx_cpu, ref["indices"])]).float()
+    same = (hit / K).mean().item()
+    assert same > (0.999 if dtype == torch.float32 else 0.97), f"mean overlap with the oracle's expert sets {same:.4f}"
     # experts: oracle on the HIP path's own indices and gates
     from flash_moe.ops.hip.flash_expert import expert_forward
 
@@ -51,6 +68,10 @@ def stagewise_check(m, w, x, K, norm, dtype):
                                gates_cpu.to(dtype).double(), token_chunk=256)
     fro = rel_fro(e_hip, e_ref)
     assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 1e-3}[dtype], f"experts: {fro:.3e}"
+    # block output against a float64 evaluation of MLP + experts on the HIP path's own routing: only the
+    # HIP path's two roundings (the [T,I] activation and the result) remain, so the bar holds everywhere
+    y64 = orc.mlp_forward(x.view(-1, H).double(), w.gate_proj.double(), w.up_proj.double(), w.down_proj.double()) + e_hip.double()
+    assert_output_close(y.view(-1, H), y64.to(dtype), dtype, "block output vs float64 oracle")
     return same
 
 
@@ -59,8 +80,7 @@ def test_block_c1_fp32(norm):
     # C1: fp32, 1 x 512 tokens, H=256, I=1024, E=1024 (32x32 keys), K=16
     m, w = build(256, 1024, 1024, 16, norm, torch.float32)
     x = torch.randn(1, 512, 256, generator=torch.Generator().manual_seed(0))
-    same = stagewise_check(m, w, x, 16, norm, torch.float32)
-    assert same > 0.97
+    stagewise_check(m, w, x, 16, norm, torch.float32)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
