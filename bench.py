@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the FlashMoE forward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one forward pass of the FlashMoE block (README configuration: bf16, batch 1 x seq 4096,
+hidden 1024, intermediate 4096, 16384 experts, top-64, norm_topk_prob False) over one synthetic batch
+that is already resident in HBM.  The last line printed is one JSON object:
+
+  value          tokens/s of the whole block (4096 tokens / mean step time over K steps)
+  stages         mean duration of each launch of the block, measured with HIP events on the launch stream
+  roofline       the slowest kernel of the block against the roofline that bounds it
+  expert_c3      the routed-expert kernel alone on its own benchmark shape (16384 tokens), as HBM GB/s
+  cpu_baseline   the CPU restatement of the reference's eager path (oracle/) on the same block, timed on
+                 this machine's host cores
+
+Only one GPU is used; --gpus N with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "flash-moe_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+C4 = dict(batch=1, seq=4096, hidden=1024, inter=4096, experts=16384, top_k=64, norm=False)
+C3 = dict(tokens=16384, hidden=1024, experts=16384, top_k=64)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def synthetic_block(cfg, dtype, device):
+    """FlashMoE module with seeded N(0, 0.02) weights and a seeded N(0, 1) input."""
+    import torch
+
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+
+    g = torch.Generator(device="cpu").manual_seed(0)
+    m = FlashMoE(FlashMoEConfig(cfg["hidden"], cfg["inter"], "silu", cfg["experts"], cfg["top_k"], cfg["norm"]))
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.02)
+    x = torch.randn(cfg["batch"], cfg["seq"], cfg["hidden"], generator=g)
+    return m.to(device=device, dtype=dtype), x.to(device=device, dtype=dtype)
+
+
+def event_time_ms(fn, iters, warmup=3):
+    """Mean duration of fn() over `iters` back-to-back calls, from HIP events on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def expert_bytes(T, H, K, touched, elt):
+    """Algorithmic bytes of the routed-expert op: x in and out, each touched down/up row once,
+    int64 indices and gates."""
+    return 2 * T * H * elt + 2 * touched * H * elt + T * K * (8 + elt)
+
+
+def stage_kernels(m, x):
+    """Callables that launch exactly one stage each through the C ABI (no allocation inside)."""
+    import torch
+
+    from flash_moe import _C
+
+    L = _C.lib()
+    dev = x.device
+    stream = lambda: _C.current_stream(dev)
+    tokens = x.view(-1, m.hidden_size)
+    T, H, I, K, nk = tokens.shape[0], m.hidden_size, m.intermediate_size, m.top_k, m.num_keys
+    code = _C.dtype_code(x.dtype)
+    was_training = m.training
+    m.eval()
+    with torch.no_grad():
+        _, lp = m.router_log_probs(tokens)
+    m.train(was_training)
+    lp = lp.contiguous()
+    scores = torch.empty(T, K, device=dev, dtype=torch.float32)
+    indices = torch.empty(T, K, device=dev, dtype=torch.int64)
+    gates32 = torch.empty(T, K, device=dev, dtype=torch.float32)
+    L.fmoe_router_topk(lp.data_ptr(), T, nk, K, _C.F32, scores.data_ptr(), indices.data_ptr(), gates32.data_ptr(),
+                       int(m.norm_topk_prob), stream())
+    gates = gates32.to(x.dtype)
+    experts = torch.empty_like(tokens)
+    act = torch.empty(T, I, device=dev, dtype=x.dtype)
+    out = torch.empty_like(tokens)
+    wd_t, wu_t = m.down_embed.weight, m.up_embed.weight
+    E = wd_t.shape[0]
+    ws_bytes = L.fmoe_expert_workspace_bytes(T, H, E, K, code)
+    ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(L.fmoe_last_error().decode())
+
+    fns = {
+        "router_topk": lambda: check(L.fmoe_router_topk(lp.data_ptr(), T, nk, K, _C.F32, scores.data_ptr(),
+                                                        indices.data_ptr(), gates32.data_ptr(),
+                                                        int(m.norm_topk_prob), stream())),
+        "expert": lambda: check(L.fmoe_expert_forward(tokens.data_ptr(), wd_t.data_ptr(), wu_t.data_ptr(),
+                                                      indices.data_ptr(), gates.data_ptr(), T, H, E, K, code,
+                                                      experts.data_ptr(), ws.data_ptr(), ws_bytes, stream())),
+        "mlp_gate_up": lambda: check(L.fmoe_mlp_gate_up(tokens.data_ptr(), m.gate_proj.weight.data_ptr(),
+                                                        m.up_proj.weight.data_ptr(), T, H, I, code, act.data_ptr(),
+                                                        stream())),
+        "mlp_down": lambda: check(L.fmoe_mlp_down(act.data_ptr(), m.down_proj.weight.data_ptr(), T, H, I, code,
+                                                  experts.data_ptr(), out.data_ptr(), stream())),
+    }
+    with torch.no_grad():
+        prologue = lambda: m.router_log_probs(tokens)
+    touched = int(torch.unique(indices).numel())
+    elt = x.element_size()
+    work = {
+        "router_topk": dict(bound="hbm", bytes=2 * T * nk * 4 + T * K * (4 + 8 + 4)),
+        "expert": dict(bound="hbm", bytes=expert_bytes(T, H, K, touched, elt), touched_experts=touched),
+        "mlp_gate_up": dict(bound="mfma", flops=2 * T * H * 2 * I),
+        "mlp_down": dict(bound="mfma", flops=2 * T * I * H),
+    }
+    keep = (lp, scores, indices, gates32, gates, experts, act, out, ws)
+    return fns, prologue, work, keep
+
+
+def roofline_entry(name, ms, w, traffic):
+    if w["bound"] == "hbm":
+        achieved = w["bytes"] / (ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = w["flops"] / (ms * 1e-3) / 1e12
+        peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    return dict(kernel=name, bound=w["bound"], achieved=round(achieved, 2), peak=peak, unit=unit,
+                frac=round(achieved / peak, 4), avg_launch_us=round(ms * 1e3, 2),
+                algorithmic=w.get("bytes", w.get("flops")), traffic=traffic)
+
+
+def measured_traffic(kernel, workload):
+    """HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, if a summary is committed."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(workload, {}).get(kernel)
+    except (OSError, ValueError):
+        return None
+
+
+def bench_expert_c3(dtype, iters):
+    import torch
+
+    from flash_moe import _C
+
+    cfg = C3
+    T, H, E, K = cfg["tokens"], cfg["hidden"], cfg["experts"], cfg["top_k"]
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(T, H, generator=g).to(dtype).cuda()
+    wd = (torch.randn(E, H, generator=g) * 0.02).to(dtype).cuda()
+    wu = (torch.randn(E, H, generator=g) * 0.02).to(dtype).cuda()
+    gidx = torch.Generator(device="cuda").manual_seed(0)
+    idx = torch.rand(T, E, device="cuda", generator=gidx).topk(K, dim=-1).indices.contiguous()   # K distinct ids per token
+    gates = torch.softmax(torch.randn(T, K, generator=g), -1).to(dtype).cuda()
+    out = torch.empty_like(x)
+    L = _C.lib()
+    code = _C.dtype_code(dtype)
+    ws_bytes = L.fmoe_expert_workspace_bytes(T, H, E, K, code)
+    ws = torch.empty(max(ws_bytes, 1), device="cuda", dtype=torch.uint8)
+    stream = lambda: _C.current_stream(x.device)
+
+    def run():
+        rc = L.fmoe_expert_forward(x.data_ptr(), wd.data_ptr(), wu.data_ptr(), idx.data_ptr(), gates.data_ptr(), T, H,
+                                   E, K, code, out.data_ptr(), ws.data_ptr(), ws_bytes, stream())
+        if rc:
+            raise RuntimeError(L.fmoe_last_error().decode())
+
+    ms = event_time_ms(run, iters)
+    touched = int(torch.unique(idx).numel())
+    nbytes = expert_bytes(T, H, K, touched, x.element_size())
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return dict(workload=f"expert kernel only: bf16, {T} tokens, hidden {H}, {E} experts, top-{K}, distinct ids per token",
+                avg_launch_us=round(ms * 1e3, 2), algorithmic_bytes=nbytes, touched_experts=touched,
+                achieved_GBps=round(gbs, 1), peak_GBps=HBM_PEAK_GBS, frac=round(gbs / HBM_PEAK_GBS, 4),
+                tokens_per_s=round(T / (ms * 1e-3)), traffic=measured_traffic("expert", "c3"))
+
+
+def cpu_baseline(cfg, dtype, budget_s=20.0):
+    """The oracle's block forward on the same workload, on the host cores (checker timed as a baseline)."""
+    import torch
+
+    from oracle import flashmoe_oracle as orc
+
+    threads = torch.get_num_threads()
+    w = orc.make_block_weights(cfg["hidden"], cfg["inter"], cfg["experts"], seed=0).to(dtype)
+    x = torch.randn(cfg["batch"], cfg["seq"], cfg["hidden"], generator=torch.Generator().manual_seed(0)).to(dtype)
+    T = cfg["batch"] * cfg["seq"]
+    times = []
+    t_begin = time.perf_counter()
+    with torch.no_grad():
+        orc.block_forward(x, w, cfg["top_k"], cfg["norm"], token_chunk=512)   # warm-up
+        while len(times) < 5 or (time.perf_counter() - t_begin < budget_s and len(times) < 50):
+            t0 = time.perf_counter()
+            orc.block_forward(x, w, cfg["top_k"], cfg["norm"], token_chunk=512)
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - t_begin > 3 * budget_s:
+                break
+    med = statistics.median(times)
+    return dict(value=round(T / med, 1), unit="tokens/s", cores=threads, kind="port",
+                sample=f"whole C4 batch ({T} tokens, {str(dtype).replace('torch.', '')}), median of {len(times)} "
+                       f"forward passes of the torch CPU restatement of FlashMoE_Pytorch.forward, {threads} threads",
+                ms_per_step=round(med * 1e3, 2))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-c3", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (the forward path is single-GPU; "
+              "see DESIGN.md for how it would shard)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        sys.exit(1)
+    from flash_moe import _C
+
+    _C.lib()   # fail loudly here if the HIP library is missing
+    dtype = torch.bfloat16
+    torch.cuda.set_device(0)
+    m, x = synthetic_block(C4, dtype, "cuda:0")
+    T = C4["batch"] * C4["seq"]
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            m(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            m(x)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    log(f"block: {ms_per_step:.3f} ms/step -> {T / ms_per_step * 1e3:.0f} tokens/s")
+
+    # per-stage durations (HIP events on the launch stream), kernels launched through the C ABI
+    fns, prologue, work, keep = stage_kernels(m, x)
+    iters = max(20, min(200, args.steps))
+    stages = {}
+    with torch.no_grad():
+        stages["router_prologue_torch"] = round(event_time_ms(prologue, iters) * 1e3, 2)
+    times = {}
+    for name, fn in fns.items():
+        times[name] = event_time_ms(fn, iters)
+        stages[name] = round(times[name] * 1e3, 2)
+    log("stage durations (us):", stages)
+    rooflines = {n: roofline_entry(n, times[n], work[n], measured_traffic(n, "c4")) for n in fns}
+    dominant = max(times, key=times.get)
+
+    result = {
+        "metric": "FlashMoE fwd tokens/s (h1024, 16K experts, top-64)",
+        "value": round(T / ms_per_step * 1e3, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C4 full FlashMoE block (README config): bf16, batch 1 x seq 4096, hidden 1024, "
+                               "intermediate 4096, silu, 16384 experts, top-64, norm_topk_prob False, train-mode batch norm",
+                   "tokens": T, "hidden": C4["hidden"], "intermediate": C4["inter"], "num_experts": C4["experts"],
+                   "top_k": C4["top_k"]},
+        "roofline": rooflines[dominant],
+        "stages_us": stages,
+        "rooflines_all": rooflines,
+    }
+    if not args.no_c3:
+        result["expert_c3"] = bench_expert_c3(dtype, max(10, min(50, args.steps)))
+        log("expert C3:", result["expert_c3"])
+    del keep
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(C4, dtype)
+        log("cpu baseline:", result["cpu_baseline"])
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -272,34 +272,49 @@ void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, 
 }
 
 template <typename T>
-int mlp_16bit(const void* x, const void* wg, const void* wu, const void* wd, int64_t T_, int H, int I,
-              const void* residual, void* out, void* h, hipStream_t stream) {
-    const int M = (int)T_;
-    // gate/up: N = I output columns; down: N = H.  Large tiles when they still give every CU work.
-    const int64_t big_tiles_1 = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
-    if (big_tiles_1 >= 256)
+int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, hipStream_t stream) {
+    // N = I output columns.  Large tiles when they still give every CU work.
+    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
+    if (big_tiles >= 256)
         launch_gemm<T, 256, 256, kEpiSwiGLU>((const T*)x, (const T*)wg, (const T*)wu, (T*)h, nullptr, M, I, H, stream);
     else
         launch_gemm<T, 128, 128, kEpiSwiGLU>((const T*)x, (const T*)wg, (const T*)wu, (T*)h, nullptr, M, I, H, stream);
-    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(gate/up)");
-    const int64_t big_tiles_2 = (int64_t)((M + 255) / 256) * ((H + 255) / 256);
-    if (big_tiles_2 >= 256)
-        launch_gemm<T, 256, 256, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
-    else
-        launch_gemm<T, 128, 128, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
-    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(down)");
+    FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up)");
     return FMOE_OK;
 }
 
-int mlp_f32(const void* x, const void* wg, const void* wu, const void* wd, int64_t T_, int H, int I,
-            const void* residual, void* out, void* h, hipStream_t stream) {
-    const int M = (int)T_;
+template <typename T>
+int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
+    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((H + 255) / 256);
+    if (big_tiles >= 256)
+        launch_gemm<T, 256, 256, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
+    else
+        launch_gemm<T, 128, 128, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
+    FMOE_CHECK_LAUNCH("fmoe_mlp(down)");
+    return FMOE_OK;
+}
+
+int gate_up_f32(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, hipStream_t stream) {
     hipLaunchKernelGGL((sgemm_nt_kernel<kEpiSwiGLU>), dim3((I + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
                        (const float*)x, (const float*)wg, (const float*)wu, (float*)h, nullptr, M, I, H);
-    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(gate/up, f32)");
+    FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up, f32)");
+    return FMOE_OK;
+}
+
+int down_f32(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
     hipLaunchKernelGGL((sgemm_nt_kernel<kEpiPlain>), dim3((H + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
                        (const float*)h, (const float*)wd, nullptr, (float*)out, (const float*)residual, M, H, I);
-    FMOE_CHECK_LAUNCH("fmoe_mlp_forward(down, f32)");
+    FMOE_CHECK_LAUNCH("fmoe_mlp(down, f32)");
+    return FMOE_OK;
+}
+
+int check_mlp_shape(const char* who, int64_t T_, int H, int I, int dtype) {
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "%s: unknown dtype %d", who, dtype);
+    FMOE_REQUIRE(T_ >= 0 && H > 0 && I > 0, FMOE_ERR_BAD_SHAPE, "%s: bad shape T=%lld H=%d I=%d", who, (long long)T_, H, I);
+    FMOE_REQUIRE(T_ < (1ll << 31), FMOE_ERR_UNSUPPORTED, "%s: T=%lld >= 2^31", who, (long long)T_);
+    if (dtype != FMOE_F32)
+        FMOE_REQUIRE(H % 8 == 0 && I % 8 == 0, FMOE_ERR_ALIGNMENT,
+                     "%s: hidden=%d and intermediate=%d must be multiples of 8 (16-byte rows)", who, H, I);
     return FMOE_OK;
 }
 
@@ -312,32 +327,53 @@ extern "C" size_t fmoe_mlp_workspace_bytes(int64_t num_tokens, int hidden, int i
     return fmoe::round_up((size_t)num_tokens * (size_t)intermediate * fmoe::dtype_size(dtype), 256);
 }
 
+extern "C" int fmoe_mlp_gate_up(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
+                                int intermediate, int dtype, void* act, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    if (int rc = check_mlp_shape("fmoe_mlp_gate_up", num_tokens, hidden, intermediate, dtype)) return rc;
+    if (num_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(x && gate_w && up_w && act, FMOE_ERR_NULL_POINTER, "fmoe_mlp_gate_up: null tensor pointer");
+    FMOE_REQUIRE(dtype == FMOE_F32 || (aligned16(x) && aligned16(gate_w) && aligned16(up_w) && aligned16(act)),
+                 FMOE_ERR_ALIGNMENT, "fmoe_mlp_gate_up: tensor pointers must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const int M = (int)num_tokens;
+    switch (dtype) {
+        case FMOE_F32: return gate_up_f32(x, gate_w, up_w, M, hidden, intermediate, act, s);
+        case FMOE_BF16: return gate_up_16bit<bf16_t>(x, gate_w, up_w, M, hidden, intermediate, act, s);
+        default: return gate_up_16bit<f16_t>(x, gate_w, up_w, M, hidden, intermediate, act, s);
+    }
+}
+
+extern "C" int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int hidden, int intermediate,
+                             int dtype, const void* residual, void* out, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    if (int rc = check_mlp_shape("fmoe_mlp_down", num_tokens, hidden, intermediate, dtype)) return rc;
+    if (num_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(act && down_w && out, FMOE_ERR_NULL_POINTER, "fmoe_mlp_down: null tensor pointer");
+    FMOE_REQUIRE(dtype == FMOE_F32 || (aligned16(act) && aligned16(down_w)), FMOE_ERR_ALIGNMENT,
+                 "fmoe_mlp_down: tensor pointers must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const int M = (int)num_tokens;
+    switch (dtype) {
+        case FMOE_F32: return down_f32(act, down_w, M, hidden, intermediate, residual, out, s);
+        case FMOE_BF16: return down_16bit<bf16_t>(act, down_w, M, hidden, intermediate, residual, out, s);
+        default: return down_16bit<f16_t>(act, down_w, M, hidden, intermediate, residual, out, s);
+    }
+}
+
 extern "C" int fmoe_mlp_forward(const void* x, const void* gate_w, const void* up_w, const void* down_w,
                                 int64_t num_tokens, int hidden, int intermediate, int dtype, const void* residual,
                                 void* out, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace fmoe;
     clear_error();
-    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_mlp_forward: unknown dtype %d", dtype);
-    FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && intermediate > 0, FMOE_ERR_BAD_SHAPE,
-                 "fmoe_mlp_forward: bad shape T=%lld H=%d I=%d", (long long)num_tokens, hidden, intermediate);
-    FMOE_REQUIRE(num_tokens < (1ll << 31), FMOE_ERR_UNSUPPORTED, "fmoe_mlp_forward: T=%lld >= 2^31",
-                 (long long)num_tokens);
+    if (int rc = check_mlp_shape("fmoe_mlp_forward", num_tokens, hidden, intermediate, dtype)) return rc;
     if (num_tokens == 0) return FMOE_OK;
     FMOE_REQUIRE(x && gate_w && up_w && down_w && out, FMOE_ERR_NULL_POINTER, "fmoe_mlp_forward: null tensor pointer");
     const size_t need = fmoe_mlp_workspace_bytes(num_tokens, hidden, intermediate, dtype);
     FMOE_REQUIRE(workspace && workspace_bytes >= need, FMOE_ERR_WORKSPACE,
                  "fmoe_mlp_forward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-    if (dtype != FMOE_F32) {
-        FMOE_REQUIRE(hidden % 8 == 0 && intermediate % 8 == 0, FMOE_ERR_ALIGNMENT,
-                     "fmoe_mlp_forward: hidden=%d and intermediate=%d must be multiples of 8 (16-byte rows)", hidden,
-                     intermediate);
-        FMOE_REQUIRE(aligned16(x) && aligned16(gate_w) && aligned16(up_w) && aligned16(down_w) && aligned16(workspace),
-                     FMOE_ERR_ALIGNMENT, "fmoe_mlp_forward: tensor pointers must be 16-byte aligned");
-    }
-    hipStream_t s = (hipStream_t)stream;
-    switch (dtype) {
-        case FMOE_F32: return mlp_f32(x, gate_w, up_w, down_w, num_tokens, hidden, intermediate, residual, out, workspace, s);
-        case FMOE_BF16: return mlp_16bit<bf16_t>(x, gate_w, up_w, down_w, num_tokens, hidden, intermediate, residual, out, workspace, s);
-        default: return mlp_16bit<f16_t>(x, gate_w, up_w, down_w, num_tokens, hidden, intermediate, residual, out, workspace, s);
-    }
+    if (int rc = fmoe_mlp_gate_up(x, gate_w, up_w, num_tokens, hidden, intermediate, dtype, workspace, stream)) return rc;
+    return fmoe_mlp_down(workspace, down_w, num_tokens, hidden, intermediate, dtype, residual, out, stream);
 }

@@ -103,6 +103,18 @@ int fmoe_mlp_forward(const void* x, const void* gate_w, const void* up_w, const 
                      int64_t num_tokens, int hidden, int intermediate, int dtype, const void* residual,
                      void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The two launches of fmoe_mlp_forward, individually (same argument rules; `act` is the [T,I] activation
+ * that fmoe_mlp_forward keeps in its workspace).  A caller that wants the activation, or that times
+ * the two GEMMs separately, calls these instead.
+ *   fmoe_mlp_gate_up: act = silu(x gate_w^T) * (x up_w^T)     -- the two matmuls and the SwiGLU kernel of
+ *                     triton_flash_mlp_func (flash_moe/ops/triton/flash_mlp.py:175-179, 25-49)
+ *   fmoe_mlp_down:    out = act down_w^T [+ residual]          -- its last matmul (flash_mlp.py:173-181) */
+int fmoe_mlp_gate_up(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
+                     int intermediate, int dtype, void* act, void* stream);
+
+int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int hidden, int intermediate, int dtype,
+                  const void* residual, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
