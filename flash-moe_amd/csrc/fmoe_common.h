@@ -74,10 +74,27 @@ template <typename T> __device__ inline float round_through(float v) { return El
 // ---- wave64 helpers --------------------------------------------------------------------------
 __device__ inline int lane_id() { return (int)(threadIdx.x & (kWave - 1)); }
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+// Cross-lane moves through the DPP path (no LDS traffic).  CTRL: 0xB1 / 0x4E = swap lanes 1 / 2 apart inside
+// a quad, 0x141 = mirror inside 8 lanes, 0x140 = mirror inside a row of 16 lanes, 0x128 = rotate a row by 8
+// (= swap lanes 8 apart), 0x142 / 0x143 = broadcast lane 15 / 31 to the following row(s).
+template <int CTRL, int ROW_MASK = 0xF, bool BOUND = true>
+__device__ inline float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, BOUND));
+}
+// Sum over each aligned group of 8 lanes, result in all 8.
+__device__ inline float group8_sum(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
     return v;
+}
+// Sum over the 64 lanes, result in all lanes (it comes back through an SGPR, so it is wave-uniform).
+__device__ inline float wave_sum(float v) {
+    v = group8_sum(v);
+    v += dpp_move<0x140>(v);
+    v += dpp_move<0x142, 0xA, false>(v);   // row_bcast15: lane 15 of rows 0 and 2 into rows 1 and 3
+    v += dpp_move<0x143, 0xC, false>(v);   // row_bcast31: lane 31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 __device__ inline float silu_f32(float v) { return v / (1.0f + __expf(-v)); }

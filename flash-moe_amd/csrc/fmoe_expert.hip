@@ -159,9 +159,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
             s[u] = part;
         }
 #pragma unroll
-        for (int m = 32; m >= 1; m >>= 1)
-#pragma unroll
-            for (int u = 0; u < kPairsInFlight; ++u) s[u] += __shfl_xor(s[u], m, kWave);
+        for (int u = 0; u < kPairsInFlight; ++u) s[u] = wave_sum(s[u]);
 #pragma unroll
         for (int u = 0; u < kPairsInFlight; ++u) {
             const float a = silu_f32(s[u]) * gate[u];
@@ -178,7 +176,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
 }
 
 template <typename T>
-int launch_expert(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
+int launch_expert_rows(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
                   int64_t T_, int H, int64_t E, int K, void* out, hipStream_t stream) {
     constexpr int V = Elem<T>::kVec;
     const int packets = H / V;
@@ -202,23 +200,277 @@ int launch_expert(const void* x, const void* down, const void* up, const int64_t
     return FMOE_OK;
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Column-slice path.
+//
+// Random 2 KiB row gathers from tables of tens of MiB are served by the Infinity Cache / HBM through the
+// fabric at ~7.6 TB/s on MI355X whatever the kernel does, while gathers from a working set that fits one
+// XCD's 4 MiB L2 run at ~25 TB/s.  So the tables are processed in column slices of 128 bytes (one L2
+// line per row): a slice of a 16384-row table is 2 MiB.  Workgroups are mapped so that XCD x works on
+// slices x, x+8, ... one after the other (workgroup ids are dealt round-robin over the 8 XCDs), each
+// slice streaming through all tokens while its 2 MiB stay resident in that XCD's L2; every table byte
+// leaves HBM / Infinity Cache once.  A wave-wide load fetches the 128-byte pieces of 8 different pairs
+// (8 lanes x 16 bytes each); 8 such loads are in flight per wave.
+//
+//   prepare : int64 ids -> int32 (-1 if outside [0,E))
+//   scores  : spart[slice][pair] = <x[token, slice cols], down[expert, slice cols]>          (per slice)
+//   gate    : a[pair] = silu(sum_slice spart[slice][pair]) * gate[pair]
+//   states  : out[token, slice cols] = sum_k a[token,k] * up[expert_k, slice cols]           (per slice)
+// `states` needs no cross-slice reduction, so the output is still written exactly once, without atomics.
+// ------------------------------------------------------------------------------------------------
+constexpr int kChunkLanes = 8;     // lanes covering one 128-byte chunk
+constexpr int kChunkPairs = 8;     // pairs per wave-wide load
+constexpr int kSliceLoads = 8;     // wave-wide loads in flight: 64 pairs per round
+constexpr uint32_t kBadOffset = 0xFFF00000u;   // row offset of an invalid id: beyond any table the slice path accepts
+
+// Table rows are addressed through a raw buffer resource: 32-bit byte offsets (no 64-bit address arithmetic
+// per load) and hardware bounds checking, so the row of an invalid id reads as zeros.
+__device__ inline __amdgpu_buffer_rsrc_t table_resource(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ inline u32x4_t load_row_piece(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset) {
+    return __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0));
+}
+
+// ids -> byte offset of the row (kBadOffset if the id is outside [0,E))
+__global__ __launch_bounds__(256) void expert_prepare_kernel(const int64_t* __restrict__ idx, uint32_t* __restrict__ off32,
+                                                             int64_t n, int64_t num_experts, uint32_t row_bytes) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int64_t e = idx[i];
+        off32[i] = (e >= 0 && e < num_experts) ? (uint32_t)e * row_bytes : kBadOffset;
+    }
+}
+
+__device__ inline bool slice_of_block(int num_slices, int blocks_per_slice, int& slice, int& tb) {
+    const int b = (int)blockIdx.x;
+    const int j = b >> 3;
+    slice = (b & 7) + 8 * (j / blocks_per_slice);
+    tb = j % blocks_per_slice;
+    return slice < num_slices;
+}
+
+// p[u] holds, in each of the 8 lanes of a chunk group, that lane's share of pair u's dot product.  Returns in
+// lane c of the group the complete sum of pair u == c: a transposing butterfly (7 cross-lane adds instead of 24).
+__device__ inline float group8_transpose_sum(const float (&p)[8], int c) {
+    const bool b0 = c & 1, b1 = c & 2, b2 = c & 4;
+    float q[4], r[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float keep = b0 ? p[2 * i + 1] : p[2 * i], send = b0 ? p[2 * i] : p[2 * i + 1];
+        q[i] = keep + dpp_move<0xB1>(send);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float keep = b1 ? q[2 * i + 1] : q[2 * i], send = b1 ? q[2 * i] : q[2 * i + 1];
+        r[i] = keep + dpp_move<0x4E>(send);
+    }
+    const float keep = b2 ? r[1] : r[0], send = b2 ? r[0] : r[1];
+    return keep + __shfl_xor(send, 4, kWave);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void expert_scores_slice_kernel(
+    const T* __restrict__ x, const T* __restrict__ down, uint32_t table_bytes, const uint32_t* __restrict__ off32,
+    float* __restrict__ spart, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
+    int tokens_per_block) {
+    constexpr int V = Elem<T>::kVec;
+    int slice, tb;
+    if (!slice_of_block(num_slices, blocks_per_slice, slice, tb)) return;
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int c = lane & (kChunkLanes - 1), pg = lane >> 3;
+    const int col = slice * (kChunkLanes * V) + c * V;
+    const bool col_ok = col < hidden;                       // false only in a partial last slice
+    const uint32_t col_bytes = col_ok ? (uint32_t)col * sizeof(T) : 0u;
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    const __amdgpu_buffer_rsrc_t rsrc = table_resource(down, table_bytes);
+    const int64_t pairs = num_tokens * top_k;
+    const int64_t t_begin = (int64_t)tb * tokens_per_block;
+    const int64_t t_end = t_begin + tokens_per_block < num_tokens ? t_begin + tokens_per_block : num_tokens;
+    float* my_spart = spart + (int64_t)slice * pairs;
+
+    for (int64_t t = t_begin + wave; t < t_end; t += 4) {
+        const u32x4_t xq = col_ok ? *reinterpret_cast<const u32x4_t*>(x + t * hidden + col) : zero4;
+        const uint32_t* tok_off = off32 + t * top_k;
+        for (int k0 = 0; k0 < top_k; k0 += kWave) {
+            // one coalesced load brings the row offsets of 64 pairs; lane (pg, c) then needs those of pairs u*8+pg
+            const uint32_t mine = k0 + lane < top_k ? tok_off[k0 + lane] : kBadOffset;
+            u32x4_t w[kSliceLoads];
+#pragma unroll
+            for (int u = 0; u < kSliceLoads; ++u) {
+                const uint32_t o = (uint32_t)__builtin_amdgcn_ds_bpermute((u * kChunkPairs + pg) * 4, (int)mine);
+                w[u] = load_row_piece(rsrc, o + col_bytes);
+            }
+            float part[kSliceLoads];
+#pragma unroll
+            for (int u = 0; u < kSliceLoads; ++u) part[u] = dot16<T>(xq, w[u], 0.0f);
+            const float total = group8_transpose_sum(part, c);     // pair k0 + c*8 + pg
+            const int kk = k0 + c * kChunkPairs + pg;
+            if (kk < top_k) my_spart[t * top_k + kk] = total;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void expert_gate_kernel(const float* __restrict__ spart, const T* __restrict__ gates,
+                                                          const uint32_t* __restrict__ off32, float* __restrict__ a,
+                                                          int64_t pairs, int num_slices) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pairs) return;
+    float s = 0.0f;
+    for (int sl = 0; sl < num_slices; ++sl) s += spart[(int64_t)sl * pairs + p];
+    a[p] = off32[p] != kBadOffset ? silu_f32(s) * Elem<T>::to_f32(gates[p]) : 0.0f;
+}
+
+// acc[0..kVec) += a0 * w0 + a1 * w1 for two 16-byte packets of two different rows
+template <typename T> __device__ inline void axpy16_pair(float a0, float a1, u32x4_t w0, u32x4_t w1, float* acc) {
+    axpy16<T>(a0, w0, acc);
+    axpy16<T>(a1, w1, acc);
+}
+// bf16: interleave the two rows column by column and use the packed dot product, (w0[c], w1[c]) . (a0, a1);
+// half the instructions of unpack + fma.  The two coefficients are rounded to bf16 for this (the reference
+// forms silu(s)*g in the activation dtype as well, flash_expert.py:191).
+template <> __device__ inline void axpy16_pair<bf16_t>(float a0, float a1, u32x4_t w0, u32x4_t w1, float* acc) {
+    const bf16x2_t ap = {(bf16_t)a0, (bf16_t)a1};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t p0 = w0[i], p1 = w1[i];
+        const uint32_t lo = __builtin_amdgcn_perm(p1, p0, 0x05040100u);   // (p0.lo16, p1.lo16)
+        const uint32_t hi = __builtin_amdgcn_perm(p1, p0, 0x07060302u);   // (p0.hi16, p1.hi16)
+        acc[2 * i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, lo), ap, acc[2 * i], false);
+        acc[2 * i + 1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, hi), ap, acc[2 * i + 1], false);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void expert_states_slice_kernel(
+    const float* __restrict__ a, const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ off32,
+    T* __restrict__ out, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
+    int tokens_per_block) {
+    constexpr int V = Elem<T>::kVec;
+    int slice, tb;
+    if (!slice_of_block(num_slices, blocks_per_slice, slice, tb)) return;
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int c = lane & (kChunkLanes - 1), pg = lane >> 3;
+    const int col = slice * (kChunkLanes * V) + c * V;
+    const bool col_ok = col < hidden;
+    const uint32_t col_bytes = col_ok ? (uint32_t)col * sizeof(T) : 0u;
+    const __amdgpu_buffer_rsrc_t rsrc = table_resource(up, table_bytes);
+    const int64_t t_begin = (int64_t)tb * tokens_per_block;
+    const int64_t t_end = t_begin + tokens_per_block < num_tokens ? t_begin + tokens_per_block : num_tokens;
+
+    for (int64_t t = t_begin + wave; t < t_end; t += 4) {
+        const uint32_t* tok_off = off32 + t * top_k;
+        const float* tok_a = a + t * top_k;
+        float acc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = 0.0f;
+        for (int k0 = 0; k0 < top_k; k0 += kWave) {
+            const bool live = k0 + lane < top_k;
+            const uint32_t mine = live ? tok_off[k0 + lane] : kBadOffset;
+            const float mine_a = live ? tok_a[k0 + lane] : 0.0f;
+            u32x4_t w[kSliceLoads];
+            float av[kSliceLoads];
+#pragma unroll
+            for (int u = 0; u < kSliceLoads; ++u) {
+                const int src = (u * kChunkPairs + pg) * 4;
+                const uint32_t o = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)mine);
+                av[u] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, mine_a)));
+                w[u] = load_row_piece(rsrc, o + col_bytes);      // zeros for an invalid id (out of bounds)
+            }
+#pragma unroll
+            for (int u = 0; u < kSliceLoads; u += 2) axpy16_pair<T>(av[u], av[u + 1], w[u], w[u + 1], acc);
+        }
+        // sum the 8 pair groups (lanes c, c+8, ..., c+56 hold the same columns)
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            acc[v] += dpp_move<0x128>(acc[v]);             // lanes 8 apart
+            acc[v] += __shfl_xor(acc[v], 16, kWave);
+            acc[v] += __shfl_xor(acc[v], 32, kWave);
+        }
+        if (pg == 0 && col_ok) *reinterpret_cast<u32x4_t*>(out + t * hidden + col) = pack16<T>(acc);
+    }
+}
+
+struct SlicePlan {
+    int num_slices, blocks_per_slice, tokens_per_block;
+    unsigned grid;
+    size_t off_idx32, off_a, off_spart, bytes;
+};
+
+SlicePlan plan_slices(int64_t T_, int H, int K, size_t elt) {
+    SlicePlan p;
+    p.num_slices = (int)((H * elt + 127) / 128);
+    const int64_t want = (T_ + 3) / 4;                       // at least one token per wave
+    p.blocks_per_slice = (int)(want < 1024 ? want : 1024);   // 256 blocks of 4 waves fill one XCD; a few rounds of them
+    p.tokens_per_block = (int)((T_ + p.blocks_per_slice - 1) / p.blocks_per_slice);
+    p.grid = (unsigned)(8 * p.blocks_per_slice * ((p.num_slices + 7) / 8));
+    const size_t pairs = (size_t)T_ * (size_t)K;
+    p.off_idx32 = 0;
+    p.off_a = round_up(p.off_idx32 + pairs * 4, 256);
+    p.off_spart = round_up(p.off_a + pairs * 4, 256);
+    p.bytes = round_up(p.off_spart + (size_t)p.num_slices * pairs * 4, 256);
+    return p;
+}
+
+template <typename T>
+int launch_expert_slices(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
+                         int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+    const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
+    char* ws = (char*)workspace;
+    uint32_t* off32 = (uint32_t*)(ws + p.off_idx32);
+    const uint32_t row_bytes = (uint32_t)(H * sizeof(T));
+    const uint32_t table_bytes = (uint32_t)(E * (int64_t)row_bytes);
+    float* a = (float*)(ws + p.off_a);
+    float* spart = (float*)(ws + p.off_spart);
+    const int64_t pairs = T_ * K;
+    const unsigned flat_grid = (unsigned)((pairs + 255) / 256);
+    hipLaunchKernelGGL(expert_prepare_kernel, dim3(flat_grid), dim3(256), 0, stream, indices, off32, pairs, E, row_bytes);
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(prepare)");
+    hipLaunchKernelGGL((expert_scores_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const T*)x, (const T*)down,
+                       table_bytes, (const uint32_t*)off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(scores)");
+    hipLaunchKernelGGL((expert_gate_kernel<T>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
+                       (const T*)gates, (const uint32_t*)off32, a, pairs, p.num_slices);
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(gate)");
+    hipLaunchKernelGGL((expert_states_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
+                       (const T*)up, table_bytes, (const uint32_t*)off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
+                       p.tokens_per_block);
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(states)");
+    return FMOE_OK;
+}
+
+// A 128-byte slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic;
+// up to 8 MiB the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
+// too few pairs to pay for four launches, whole rows are gathered by the one-wave-per-token kernel.
+bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) && T_ * K >= (1ll << 15); }
+// rows are addressed with 32-bit byte offsets below kBadOffset
+bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
+
 }  // namespace
 }  // namespace fmoe
 
-extern "C" size_t fmoe_expert_workspace_bytes(int64_t, int, int64_t, int, int) { return 0; }
-
-extern "C" int fmoe_expert_forward(const void* x, const void* down, const void* up, const int64_t* indices,
-                                   const void* gates, int64_t num_tokens, int hidden, int64_t num_experts,
-                                   int top_k, int dtype, void* out, void* workspace, size_t workspace_bytes,
-                                   void* stream) {
+extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
     using namespace fmoe;
-    (void)workspace;
-    (void)workspace_bytes;
+    (void)num_experts;
+    if (num_tokens <= 0 || hidden <= 0 || top_k <= 0 || !dtype_ok(dtype)) return 0;
+    // sized for the column-slice path whichever path a call ends up taking
+    return plan_slices(num_tokens, hidden, top_k, dtype_size(dtype)).bytes;
+}
+
+extern "C" int fmoe_expert_forward_algo(const void* x, const void* down, const void* up, const int64_t* indices,
+                                        const void* gates, int64_t num_tokens, int hidden, int64_t num_experts,
+                                        int top_k, int dtype, void* out, void* workspace, size_t workspace_bytes,
+                                        int algo, void* stream) {
+    using namespace fmoe;
     clear_error();
     FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_expert_forward: unknown dtype %d", dtype);
     FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_experts > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
                  "fmoe_expert_forward: bad shape T=%lld H=%d E=%lld K=%d", (long long)num_tokens, hidden,
                  (long long)num_experts, top_k);
+    FMOE_REQUIRE(algo >= FMOE_EXPERT_AUTO && algo <= FMOE_EXPERT_SLICES, FMOE_ERR_UNSUPPORTED,
+                 "fmoe_expert_forward: unknown algo %d", algo);
     if (num_tokens == 0) return FMOE_OK;
     FMOE_REQUIRE(x && down && up && out, FMOE_ERR_NULL_POINTER, "fmoe_expert_forward: null tensor pointer");
     FMOE_REQUIRE(top_k == 0 || (indices && gates), FMOE_ERR_NULL_POINTER,
@@ -228,10 +480,38 @@ extern "C" int fmoe_expert_forward(const void* x, const void* down, const void* 
                  "fmoe_expert_forward: hidden=%d must be a multiple of %d (16-byte rows)", hidden, vec);
     FMOE_REQUIRE(aligned16(x) && aligned16(down) && aligned16(up) && aligned16(out), FMOE_ERR_ALIGNMENT,
                  "fmoe_expert_forward: tensor pointers must be 16-byte aligned");
+    FMOE_REQUIRE(num_experts < (1ll << 31) && (int64_t)num_tokens * top_k < (1ll << 40), FMOE_ERR_UNSUPPORTED,
+                 "fmoe_expert_forward: problem too large (E=%lld, pairs=%lld)", (long long)num_experts,
+                 (long long)(num_tokens * top_k));
     hipStream_t s = (hipStream_t)stream;
-    switch (dtype) {
-        case FMOE_F32: return launch_expert<float>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
-        case FMOE_BF16: return launch_expert<bf16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
-        default: return launch_expert<f16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+    bool slices = algo == FMOE_EXPERT_SLICES || (algo == FMOE_EXPERT_AUTO && slices_pay(num_tokens, num_experts, top_k));
+    if (top_k == 0) slices = false;
+    if (slices && !slices_possible(num_experts, hidden, dtype_size(dtype))) {
+        FMOE_REQUIRE(algo == FMOE_EXPERT_AUTO, FMOE_ERR_UNSUPPORTED,
+                     "fmoe_expert_forward: tables of 4 GiB or more cannot use the column-slice schedule");
+        slices = false;
     }
+    if (slices) {
+        const size_t need = fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, dtype);
+        FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
+                     "fmoe_expert_forward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+        switch (dtype) {
+            case FMOE_F32: return launch_expert_slices<float>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            case FMOE_BF16: return launch_expert_slices<bf16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            default: return launch_expert_slices<f16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+        }
+    }
+    switch (dtype) {
+        case FMOE_F32: return launch_expert_rows<float>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+        case FMOE_BF16: return launch_expert_rows<bf16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+        default: return launch_expert_rows<f16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+    }
+}
+
+extern "C" int fmoe_expert_forward(const void* x, const void* down, const void* up, const int64_t* indices,
+                                   const void* gates, int64_t num_tokens, int hidden, int64_t num_experts,
+                                   int top_k, int dtype, void* out, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
+    return fmoe_expert_forward_algo(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dtype, out,
+                                    workspace, workspace_bytes, FMOE_EXPERT_AUTO, stream);
 }

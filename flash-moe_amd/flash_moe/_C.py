@@ -21,6 +21,8 @@ _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 
 ERR_TOPK_RANGE = -3
 
+EXPERT_AUTO, EXPERT_ROWS, EXPERT_SLICES = 0, 1, 2
+
 _vp, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
 
 # name -> (restype, argtypes); mirrors include/flashmoe_hip.h one to one
@@ -30,6 +32,7 @@ SIGNATURES = {
     "fmoe_router_topk": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
     "fmoe_expert_workspace_bytes": (_sz, [_i64, _int, _i64, _int, _int]),
     "fmoe_expert_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
+    "fmoe_expert_forward_algo": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _int, _vp]),
     "fmoe_mlp_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
     "fmoe_mlp_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_mlp_gate_up": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp]),

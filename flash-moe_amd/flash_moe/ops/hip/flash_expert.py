@@ -12,7 +12,8 @@ from flash_moe import _C
 from flash_moe.ops.utils import ensure_contiguous
 
 
-def expert_forward(hidden_states, down_weights, up_weights, indices, routing_weights) -> torch.Tensor:
+def expert_forward(hidden_states, down_weights, up_weights, indices, routing_weights, algo: int = _C.EXPERT_AUTO) -> torch.Tensor:
+    """``algo`` picks the schedule (``_C.EXPERT_AUTO`` / ``EXPERT_ROWS`` / ``EXPERT_SLICES``); the result is the same."""
     if hidden_states.dim() != 2 or down_weights.dim() != 2 or up_weights.dim() != 2:
         raise ValueError("hidden_states, down_weights and up_weights must be 2-D")
     if indices.dim() != 2 or routing_weights.shape != indices.shape:
@@ -38,9 +39,9 @@ def expert_forward(hidden_states, down_weights, up_weights, indices, routing_wei
     ws_bytes = L.fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, code)
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8) if ws_bytes else None
     with torch.cuda.device(dev):
-        status = L.fmoe_expert_forward(
+        status = L.fmoe_expert_forward_algo(
             _C.ptr(x), _C.ptr(wd), _C.ptr(wu), _C.ptr(idx), _C.ptr(g), num_tokens, hidden, num_experts, top_k,
-            code, _C.ptr(out), _C.ptr(ws), ws_bytes, _C.current_stream(dev),
+            code, _C.ptr(out), _C.ptr(ws), ws_bytes, algo, _C.current_stream(dev),
         )
     _C.check(status, "flash_expert")
     return out

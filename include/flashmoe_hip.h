@@ -61,7 +61,7 @@ const char* fmoe_last_error(void);
  *   indices    [num_tokens, top_k]        int64      i*num_keys + j; ties to the lower index (tl.argmax rule)
  *   gates      [num_tokens, top_k]        dtype      optional (NULL to skip): exp(score), divided by the
  *                                                    per-token sum when norm_topk_prob != 0
- * Requires 0 <= top_k <= num_keys (same rule as the reference's assert), num_keys <= 1024, top_k <= 256.
+ * Requires 0 <= top_k <= num_keys (same rule as the reference's assert), num_keys <= 65535, top_k <= 256.
  */
 int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
                      void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream);
@@ -85,6 +85,20 @@ size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_e
 int fmoe_expert_forward(const void* x, const void* down, const void* up, const int64_t* indices,
                         const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k,
                         int dtype, void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same operation with the schedule chosen by the caller instead of by problem size (fmoe_expert_forward
+ * passes FMOE_EXPERT_AUTO).  Both schedules compute the formula above; they differ in how the table rows
+ * travel: whole rows per (token, expert) pair, or 128-byte column slices kept resident in each XCD's L2.
+ * The reference has one schedule (expert-centric Triton kernels, flash_expert.py:580-651). */
+typedef enum {
+    FMOE_EXPERT_AUTO = 0,
+    FMOE_EXPERT_ROWS = 1,     /* one wavefront per token, whole rows; no workspace needed */
+    FMOE_EXPERT_SLICES = 2    /* column slices resident in L2; needs the workspace */
+} fmoe_expert_algo_t;
+
+int fmoe_expert_forward_algo(const void* x, const void* down, const void* up, const int64_t* indices,
+                             const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k,
+                             int dtype, void* out, void* workspace, size_t workspace_bytes, int algo, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Shared SwiGLU MLP.

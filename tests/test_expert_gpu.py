@@ -8,10 +8,13 @@ from oracle import flashmoe_oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-def run(x, wd, wu, idx, g):
-    from flash_moe.ops import flash_expert_func
+ALGOS = {"auto": 0, "rows": 1, "slices": 2}
 
-    return flash_expert_func(*cuda(x, wd, wu, idx, g)).cpu()
+
+def run(x, wd, wu, idx, g, algo="auto"):
+    from flash_moe.ops.hip.flash_expert import expert_forward
+
+    return expert_forward(*cuda(x, wd, wu, idx, g), algo=ALGOS[algo]).cpu()
 
 
 def truth64(x, wd, wu, idx, g):
@@ -19,6 +22,7 @@ def truth64(x, wd, wu, idx, g):
     return orc.expert_forward(x.double(), wd.double(), wu.double(), idx, g.double())
 
 
+@pytest.mark.parametrize("algo", ["rows", "slices"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,K", [
     (512, 256, 1024, 16),        # C1
@@ -26,11 +30,12 @@ def truth64(x, wd, wu, idx, g):
     (256, 2048, 4096, 128),      # C5 row shape
     (37, 72, 50, 5),             # ragged: rows of 9 packets, token count not a multiple of the block
     (3, 8, 4, 1),
+    (130, 1000, 300, 70),        # K not a multiple of the 64 pairs a wave handles per round; last slice partial
 ])
-def test_expert_matches_oracle(dtype, T, H, E, K):
+def test_expert_matches_oracle(dtype, T, H, E, K, algo):
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=T + K)
     x, wd, wu, g = (t.to(dtype) for t in (x, wd, wu, g))
-    got = run(x, wd, wu, idx, g)
+    got = run(x, wd, wu, idx, g, algo)
     assert got.dtype == dtype and got.shape == (T, H)
     # (1) the stated bar: against the oracle run in the same dtype
     assert_output_close(got, orc.expert_forward(x, wd, wu, idx, g), dtype, "expert vs oracle")
@@ -39,7 +44,8 @@ def test_expert_matches_oracle(dtype, T, H, E, K):
     assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 5e-4}[dtype], fro
 
 
-def test_expert_reference_test_distribution():
+@pytest.mark.parametrize("algo", ["rows", "slices"])
+def test_expert_reference_test_distribution(algo):
     # distributions of the reference's expert benchmark (tests/test_expert.py:160-175): x ~ N(0,0.5),
     # tables ~ N(0,0.1), ids drawn WITH replacement, gates ~ N(0,0.1) (negative values allowed)
     g0 = torch.Generator().manual_seed(0)
@@ -49,18 +55,22 @@ def test_expert_reference_test_distribution():
     wu = (torch.randn(E, H, generator=g0) * 0.1).bfloat16()
     idx = torch.randint(0, E, (T, K), generator=g0)
     g = (torch.randn(T, K, generator=g0) * 0.1).bfloat16()
-    got = run(x, wd, wu, idx, g)
+    got = run(x, wd, wu, idx, g, algo)
     assert rel_fro(got, truth64(x, wd, wu, idx, g)) < 4e-3
 
 
-def test_expert_properties_full_size():
+@pytest.mark.parametrize("algo", ["rows", "slices"])
+def test_expert_properties_full_size(algo):
     # C3 at full size: size-independent properties instead of a CPU evaluation of all 1M pairs
+    import functools
+
     T, H, E, K = 16384, 1024, 16384, 64
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=0)
     x, wd, wu, g = (t.bfloat16() for t in (x, wd, wu, g))
     xc, wdc, wuc, idxc, gc = cuda(x, wd, wu, idx, g)
-    from flash_moe.ops import flash_expert_func
+    from flash_moe.ops.hip.flash_expert import expert_forward
 
+    flash_expert_func = functools.partial(expert_forward, algo=ALGOS[algo])
     out = flash_expert_func(xc, wdc, wuc, idxc, gc)
     assert torch.isfinite(out).all()
     # deterministic: no atomics, so a second run is bit-identical
@@ -79,18 +89,30 @@ def test_expert_properties_full_size():
     assert rel_fro(out[sl].cpu(), truth64(x[sl], wd, wu, idx[sl], g[sl])) < 4e-3
 
 
-def test_expert_duplicates_and_single_expert():
+def test_expert_schedules_agree():
+    # the two schedules on the same inputs: same pairs, different summation order (and, for bf16, the
+    # slice schedule rounds silu(s)*g to bf16 before the packed dot product)
+    T, H, E, K = 2048, 1024, 16384, 64
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=9)
+    for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 5e-3)):
+        args = tuple(t.to(dtype) if t.is_floating_point() else t for t in (x, wd, wu, idx, g))
+        assert rel_fro(run(*args, algo="slices"), run(*args, algo="rows")) < tol
+
+
+@pytest.mark.parametrize("algo", ["rows", "slices"])
+def test_expert_duplicates_and_single_expert(algo):
     T, H, E = 64, 256, 32
     x, wd, wu, _, _ = orc.make_expert_inputs(T, H, E, 4, seed=5, std=0.2)
     e = torch.full((T, 4), 7, dtype=torch.int64)
-    one = run(x, wd, wu, e[:, :1].contiguous(), torch.ones(T, 1))
-    rep = run(x, wd, wu, e, torch.full((T, 4), 0.25))
+    one = run(x, wd, wu, e[:, :1].contiguous(), torch.ones(T, 1), algo)
+    rep = run(x, wd, wu, e, torch.full((T, 4), 0.25), algo)
     torch.testing.assert_close(rep, one, rtol=1e-5, atol=1e-7)
     s = x @ wd[7]
     torch.testing.assert_close(one, (torch.nn.functional.silu(s)).unsqueeze(-1) * wu[7], rtol=1e-4, atol=1e-6)
 
 
-def test_expert_out_of_range_ids_contribute_nothing():
+@pytest.mark.parametrize("algo", ["rows", "slices"])
+def test_expert_out_of_range_ids_contribute_nothing(algo):
     T, H, E, K = 32, 64, 16, 4
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=6, std=0.2)
     bad = idx.clone()
@@ -99,7 +121,13 @@ def test_expert_out_of_range_ids_contribute_nothing():
     g2 = g.clone()
     g2[:, 0] = 0
     g2[::2, 1] = 0
-    torch.testing.assert_close(run(x, wd, wu, bad, g), run(x, wd, wu, idx, g2), rtol=1e-6, atol=1e-8)
+    wd[0] = float("inf")   # the slice schedule reads row 0 as a stand-in for an invalid id: it must not leak
+    wu[0] = float("nan")
+    idx[idx == 0] = 1
+    bad[bad == 0] = 1
+    got = run(x, wd, wu, bad, g, algo)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got, run(x, wd, wu, idx, g2, algo), rtol=1e-6, atol=1e-8)
 
 
 def test_expert_empty_and_noncontiguous():
