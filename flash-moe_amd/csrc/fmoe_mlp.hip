@@ -1,18 +1,23 @@
 // Shared SwiGLU MLP for gfx950:  out = (silu(x Wg^T) * (x Wu^T)) Wd^T [+ residual]
 //
-// Two launches of one MFMA GEMM kernel  C[M,N] = A[M,K] * B[N,K]^T  (both operands K-contiguous, which
-// is how x, the nn.Linear weights and the [T,I] activation are laid out, so a lane's 8 consecutive k
-// values for v_mfma_f32_32x32x16 are one 16-byte LDS read):
-//   1. gate/up: the B tile holds BN/2 rows of Wg and the same BN/2 rows of Wu, so each wave owns
-//      matching gate and up accumulators and the epilogue writes silu(gate)*up, rounded once, to the
-//      [T,I] workspace.  The gate and up products never go to memory.
+// Two launches of one MFMA GEMM  C[M,N] = A[M,K] * B[N,K]^T  (both operands K-contiguous, which is how x, the
+// nn.Linear weights and the [T,I] activation are laid out, so a lane's 8 consecutive k values for
+// v_mfma_f32_32x32x16 are one 16-byte LDS read):
+//   1. gate/up: the B tile holds BN/2 rows of Wg and the same BN/2 rows of Wu, so each wave owns matching gate
+//      and up accumulators and the epilogue writes silu(gate)*up, rounded once, to the [T,I] workspace.  The gate
+//      and up products never go to memory.
 //   2. down: plain epilogue, optional residual add (the routed-expert output in the block).
-// 256 threads = 4 waves in a 2x2 arrangement, each wave (BM/2)x(BN/2) of 32x32 MFMA tiles; A and B tiles
-// go global -> registers -> LDS with the next tile's global loads issued before the current tile's
-// MFMAs; LDS rows are 128 bytes with the 16-byte chunk index XOR-ed with (row & 7) so that the 32 rows
-// a fragment read touches spread over all banks.  Workgroup ids are remapped so that each XCD (ids are
-// dealt round-robin over the 8 XCDs) works on a compact patch of the tile grid and shares A/B tiles in
-// its own L2.
+//
+// Main kernel (gemm_dma_kernel), used when the extents are multiples of the tile: tiles go global -> LDS
+// directly (global_load_lds_dwordx4, no staging registers) into NSTAGE LDS stages, issued NSTAGE-1 k-tiles
+// ahead of their use; one workgroup barrier per k-tile; 32x32x16 MFMA fragments are read with 16-byte
+// ds_reads.  An LDS row is one k-tile of one matrix row; its 16-byte chunks are XOR-swizzled with a key built
+// from the row index so that the 16 lanes the 256-byte-per-clock LDS serves per cycle hit 64 different banks.
+// Because a DMA load writes 64 consecutive chunks, the swizzle is applied on the global side: each lane fetches
+// the chunk that belongs at its LDS position.  Workgroup ids are remapped so that each XCD (ids are dealt
+// round-robin over the 8 XCDs) works on a compact patch of the tile grid and shares A/B tiles in its own L2.
+//
+// Ragged shapes take gemm_nt_kernel (register-staged, bounds-checked); fp32 takes a plain FMA kernel.
 #include "fmoe_common.h"
 
 namespace fmoe {
@@ -208,6 +213,154 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// LDS-DMA pipelined kernel.  WAVES_M x WAVES_N waves, each (BM/WAVES_M) x (BN/WAVES_N); BKT = k extent of a stage.
+// ------------------------------------------------------------------------------------------------------------
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
+    const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
+    const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n) {
+    using Frag = typename Mfma32<T>::Frag;
+    constexpr int NWAVES = WAVES_M * WAVES_N;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MF = WM / 32, NF = WN / 32;
+    constexpr int CPR = BKT / 8;                    // 16-byte chunks per LDS row
+    constexpr int RPI = 64 / CPR;                   // rows one wave-wide DMA load covers
+    constexpr int ROWS_PER_IT = NWAVES * RPI;       // rows all waves cover per DMA round
+    constexpr int STAGE = (BM + BN) * BKT;          // elements per stage
+    constexpr int KSTEPS = BKT / 16;
+    constexpr int ROW_SHIFT = (CPR == 8) ? 1 : 2;   // log2(rows per 256 bytes)
+    constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
+    constexpr int A_ROUNDS = BM / ROWS_PER_IT, B_ROUNDS = BN / ROWS_PER_IT;
+    constexpr int DMA_PER_TILE = A_ROUNDS + B_ROUNDS;
+    static_assert(BKT == 32 || BKT == 64, "stage depth");
+    static_assert(ROWS_PER_IT % 16 == 0 && BM % ROWS_PER_IT == 0 && BN % ROWS_PER_IT == 0, "DMA rounds");
+    static_assert(EPI != kEpiSwiGLU || ((BN / 2) % ROWS_PER_IT == 0 && NF % 2 == 0), "gate/up split");
+    static_assert((NSTAGE - 2) * DMA_PER_TILE < 64, "vmcnt range");
+
+    __shared__ __attribute__((aligned(1024))) T lds[NSTAGE * STAGE];
+
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN_OUT;
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    // DMA: the lane's LDS position is row (round*ROWS_PER_IT + wave*RPI + lrow), physical chunk lp; it holds the
+    // logical chunk lp ^ key(row), key(row) = (row >> ROW_SHIFT) & (CPR-1).  ROWS_PER_IT is a multiple of 16, so the
+    // key does not depend on the round and one element offset per lane serves every load.
+    const int lrow = lane / CPR, lp = lane % CPR;
+    const int key_dma = ((wave * RPI + lrow) >> ROW_SHIFT) & (CPR - 1);
+    const int lane_off = lrow * K + ((lp ^ key_dma) << 3);
+    const T* a_src = A + (int64_t)(m0 + wave * RPI) * K + lane_off;
+    const T* b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K + lane_off;
+    const T* b_src1 = (EPI == kEpiSwiGLU) ? B1 + (int64_t)(n0 + wave * RPI) * K + lane_off : nullptr;
+
+    auto issue = [&](int kt, T* stage) {
+        const int k0 = kt * BKT;
+#pragma unroll
+        for (int r = 0; r < A_ROUNDS; ++r)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(a_src + (int64_t)r * ROWS_PER_IT * K + k0),
+                (__attribute__((address_space(3))) void*)(stage + (r * ROWS_PER_IT + wave * RPI) * BKT), 16, 0, 0);
+#pragma unroll
+        for (int r = 0; r < B_ROUNDS; ++r) {
+            const T* src;
+            if (EPI == kEpiSwiGLU && r >= B_ROUNDS / 2) src = b_src1 + (int64_t)(r - B_ROUNDS / 2) * ROWS_PER_IT * K + k0;
+            else src = b_src0 + (int64_t)r * ROWS_PER_IT * K + k0;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)src,
+                (__attribute__((address_space(3))) void*)(stage + BM * BKT + (r * ROWS_PER_IT + wave * RPI) * BKT), 16, 0, 0);
+        }
+    };
+
+    f32x16_t acc[MF][NF];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int j = 0; j < NF; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // Fragment rows of a lane are (multiple of 32) + frow: the swizzle key is the same for all of them, so the
+    // address is (row base + one per-k-step offset) + an immediate per fragment.
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int key_f = (frow >> ROW_SHIFT) & (CPR - 1);
+    const int a_row_bytes = (wm * WM + frow) * BKT * (int)sizeof(T);
+    int b_row_bytes[NF];
+#pragma unroll
+    for (int j = 0; j < NF; ++j) {
+        int row;
+        if (EPI == kEpiSwiGLU) row = (j < NF / 2) ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - NF / 2) * 32;
+        else row = wn * WN + j * 32;
+        b_row_bytes[j] = (BM + row + frow) * BKT * (int)sizeof(T);
+    }
+    int pc[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) pc[ks] = ((ks * 2 + fhalf) ^ key_f) << 4;
+
+    const int k_tiles = K / BKT;
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s)
+        if (s < k_tiles) issue(s, lds + s * STAGE);
+
+    for (int kt = 0; kt < k_tiles; ++kt) {
+        // my share of tile kt has landed once at most the loads of the NSTAGE-2 younger tiles are outstanding
+        constexpr int kKeep = (NSTAGE - 2) * DMA_PER_TILE;
+        if (kt + NSTAGE - 2 < k_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (kKeep & 0xF) | ((kKeep >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_barrier();     // everyone's share landed; everyone is done reading the stage reused below
+        if (kt + NSTAGE - 1 < k_tiles) issue(kt + NSTAGE - 1, lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE);
+        const char* stage = reinterpret_cast<const char*>(lds + (kt % NSTAGE) * STAGE);
+        Frag fa[KSTEPS][MF], fb[KSTEPS][NF];
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+                fa[ks][i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + i * 32 * BKT * (int)sizeof(T));
+#pragma unroll
+            for (int j = 0; j < NF; ++j) fb[ks][j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+                for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks][i], fb[ks][j], acc[i][j]);
+    }
+
+    // D fragment layout of v_mfma_f32_32x32x*: lane l, register v holds
+    //   row = 8*(v/4) + 4*(l/32) + (v%4)   (A / M index),   col = l%32   (B / N index)
+    if (EPI == kEpiSwiGLU) {
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int j = 0; j < NF / 2; ++j) {
+                const int col = n0 + wn * (WN / 2) + j * 32 + frow;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
+                    C[(int64_t)row * N + col] = Elem<T>::from_f32(silu_f32(acc[i][j][v]) * acc[i][j + NF / 2][v]);
+                }
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int j = 0; j < NF; ++j) {
+                const int col = n0 + wn * WN + j * 32 + frow;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
+                    float r = acc[i][j][v];
+                    if (R != nullptr) r += Elem<T>::to_f32(R[(int64_t)row * N + col]);
+                    C[(int64_t)row * N + col] = Elem<T>::from_f32(r);
+                }
+            }
+    }
+}
+
 // fp32 path (parity configuration only; not a tuned kernel): 64x64 tile, 16-deep LDS slabs, 4x4 outputs
 // per thread, plain FMA.
 template <int EPI>
@@ -271,25 +424,41 @@ void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, 
                        stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
 }
 
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI>
+void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
+    constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
+    const int tiles_m = M / BM, tiles_n = N / BN_OUT;
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI>),
+                       dim3((unsigned)(tiles_m * tiles_n)), dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N,
+                       K, tiles_m, tiles_n);
+}
+
+// Tile choice: 256-wide tiles (8 waves) halve the LDS traffic per MFMA but need >= 256 of them to occupy the chip;
+// otherwise 128x128 tiles (4 waves, two workgroups per CU).
 template <typename T>
 int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, hipStream_t stream) {
-    // N = I output columns.  Large tiles when they still give every CU work.
-    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((I + 127) / 128);
-    if (big_tiles >= 256)
-        launch_gemm<T, 256, 256, kEpiSwiGLU>((const T*)x, (const T*)wg, (const T*)wu, (T*)h, nullptr, M, I, H, stream);
+    const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu;
+    const bool k_ok = H % 64 == 0;
+    if (k_ok && M % 256 == 0 && I % 128 == 0 && (int64_t)(M / 256) * (I / 128) >= 256)
+        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
+    else if (k_ok && M % 128 == 0 && I % 64 == 0)
+        launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
     else
-        launch_gemm<T, 128, 128, kEpiSwiGLU>((const T*)x, (const T*)wg, (const T*)wu, (T*)h, nullptr, M, I, H, stream);
+        launch_gemm<T, 128, 128, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up)");
     return FMOE_OK;
 }
 
 template <typename T>
 int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
-    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((H + 255) / 256);
-    if (big_tiles >= 256)
-        launch_gemm<T, 256, 256, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
+    const T *A = (const T*)h, *W = (const T*)wd, *R = (const T*)residual;
+    const bool k_ok = I % 64 == 0;
+    if (k_ok && M % 256 == 0 && H % 256 == 0 && (int64_t)(M / 256) * (H / 256) >= 256)
+        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
+    else if (k_ok && M % 128 == 0 && H % 128 == 0)
+        launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     else
-        launch_gemm<T, 128, 128, kEpiPlain>((const T*)h, (const T*)wd, nullptr, (T*)out, (const T*)residual, M, H, I, stream);
+        launch_gemm<T, 128, 128, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(down)");
     return FMOE_OK;
 }
