@@ -34,6 +34,11 @@ void clear_error();
         }                                                                              \
     } while (0)
 
+// Top-k of the router taking raw fp32 gate outputs [T, 2*nk] (log-softmax per half is done inside); defined in
+// fmoe_router.hip, used by the fused router entry point.  gates has element type `gate_dtype`.
+int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
+                              int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, hipStream_t stream);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline size_t dtype_size(int dtype) { return dtype == FMOE_F32 ? 4 : 2; }
 inline bool dtype_ok(int dtype) { return dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16; }
@@ -95,6 +100,17 @@ __device__ inline float wave_sum(float v) {
     v += dpp_move<0x142, 0xA, false>(v);   // row_bcast15: lane 15 of rows 0 and 2 into rows 1 and 3
     v += dpp_move<0x143, 0xC, false>(v);   // row_bcast31: lane 31 into rows 2 and 3
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Max over the 64 lanes, result in all lanes.
+__device__ inline float wave_max(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, kWave));
+    v = fmaxf(v, __shfl_xor(v, 32, kWave));
+    return v;
 }
 
 __device__ inline float silu_f32(float v) { return v / (1.0f + __expf(-v)); }

@@ -1,0 +1,44 @@
+// MFMA fragment types and LDS tile helpers shared by the GEMM-shaped kernels (gfx950).
+#pragma once
+
+#include "fmoe_common.h"
+
+namespace fmoe {
+
+// v_mfma_f32_32x32x16_{bf16,f16}: D[32x32] += A[32x16] * B[16x32].  Lane l supplies row l%32 of A (column l%32 of B)
+// and 8 consecutive k values chosen by l/32; it receives D[8*(v/4) + 4*(l/32) + v%4][l%32] in register v.
+template <typename T> struct Mfma32;
+template <> struct Mfma32<bf16_t> {
+    using Frag = bf16x8_t;
+    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mfma32<f16_t> {
+    using Frag = f16x8_t;
+    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// Register-staged LDS tiles: rows of 64 elements (128 bytes), 16-byte chunk index XOR-ed with (row & 7).
+constexpr int kTileK = 64;
+constexpr int kTileChunks = kTileK / 8;
+__device__ inline int swizzled_offset(int row, int chunk) { return row * kTileK + ((chunk ^ (row & 7)) << 3); }
+
+// Map the linear workgroup id to a tile so that each XCD gets a contiguous run of the tile order, and the tile order
+// walks 8 tile-rows at a time (compact patches share A and B tiles in the XCD's L2).
+__device__ inline void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int nb = (int)gridDim.x;
+    int t = (int)blockIdx.x;
+    if ((nb & 7) == 0) t = (t & 7) * (nb >> 3) + (t >> 3);
+    constexpr int GM = 8;
+    const int width = GM * tiles_n;
+    const int group = t / width;
+    const int first_m = group * GM;
+    const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+    tm = first_m + (t % width) % gsz;
+    tn = (t % width) / gsz;
+}
+
+}  // namespace fmoe

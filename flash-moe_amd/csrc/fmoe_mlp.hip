@@ -19,48 +19,16 @@
 //
 // Ragged shapes take gemm_nt_kernel (register-staged, bounds-checked); fp32 takes a plain FMA kernel.
 #include "fmoe_common.h"
+#include "fmoe_mfma.h"
 
 namespace fmoe {
 namespace {
 
 constexpr int kGemmThreads = 256;
-constexpr int BK = 64;            // k extent of an LDS tile (elements); 8 chunks of 8 elements per row
-constexpr int kChunksPerRow = BK / 8;
+constexpr int BK = kTileK;        // k extent of a register-staged LDS tile (elements)
+constexpr int kChunksPerRow = kTileChunks;
 
 enum Epilogue { kEpiSwiGLU = 0, kEpiPlain = 1 };
-
-template <typename T> struct Mfma32;
-template <> struct Mfma32<bf16_t> {
-    using Frag = bf16x8_t;
-    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct Mfma32<f16_t> {
-    using Frag = f16x8_t;
-    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
-
-__device__ inline int swizzled_offset(int row, int chunk) {   // element offset inside a [rows][BK] tile
-    return row * BK + ((chunk ^ (row & 7)) << 3);
-}
-
-// Map the linear workgroup id to a tile so that each XCD gets a contiguous run of the tile order, and
-// the tile order walks GM tile-rows at a time (compact patches share A and B tiles).
-__device__ inline void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int nb = (int)gridDim.x;
-    int t = (int)blockIdx.x;
-    if ((nb & 7) == 0) t = (t & 7) * (nb >> 3) + (t >> 3);
-    constexpr int GM = 8;
-    const int width = GM * tiles_n;
-    const int group = t / width;
-    const int first_m = group * GM;
-    const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
-    tm = first_m + (t % width) % gsz;
-    tn = (t % width) / gsz;
-}
 
 template <typename T, int BM, int BN, int EPI>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(

@@ -38,9 +38,31 @@ __device__ inline uint64_t make_key(float score, uint32_t index) {
 __device__ inline float key_score(uint64_t k) { return order_value((uint32_t)(k >> 32)); }
 __device__ inline uint32_t key_index(uint64_t k) { return ~(uint32_t)(k & 0xffffffffu); }
 
-__device__ inline uint64_t shfl_xor_u64(uint64_t v, int mask) {
-    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, kWave);
-    const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, kWave);
+// Value of lane (lane ^ mask) for mask in {1,2,4,8,16,32}, without going through LDS: DPP inside a row of 16 lanes,
+// v_permlane16_swap / v_permlane32_swap across rows.  `mask` must be a compile-time constant after inlining.
+__device__ inline uint32_t xor_lane_u32(uint32_t v, int mask, int lane) {
+    const int iv = (int)v;
+    switch (mask) {
+        case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, iv, 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+        case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, iv, 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+        case 4: {
+            int t = __builtin_amdgcn_update_dpp(0, iv, 0x104, 0xF, 0x5, false);               // row_shl:4 into banks 0,2
+            return (uint32_t)__builtin_amdgcn_update_dpp(t, iv, 0x114, 0xF, 0xA, false);      // row_shr:4 into banks 1,3
+        }
+        case 8: return (uint32_t)__builtin_amdgcn_update_dpp(0, iv, 0x128, 0xF, 0xF, true);   // row_ror:8
+        case 16: {
+            const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);   // odd rows of [0] <-> even rows of [1]
+            return (lane & 16) ? r[0] : r[1];
+        }
+        default: {
+            const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // upper half of [0] <-> lower half of [1]
+            return (lane & 32) ? r[0] : r[1];
+        }
+    }
+}
+__device__ inline uint64_t xor_lane_u64(uint64_t v, int mask, int lane) {
+    const uint32_t lo = xor_lane_u32((uint32_t)v, mask, lane);
+    const uint32_t hi = xor_lane_u32((uint32_t)(v >> 32), mask, lane);
     return ((uint64_t)hi << 32) | lo;
 }
 
@@ -65,13 +87,12 @@ __device__ inline void bitonic_layer(uint64_t (&v)[RK], int lane, int k, int j) 
 #pragma unroll
         for (int r = 0; r < RK; ++r) {
             const int p = lane * RK + r;
-            const uint64_t other = shfl_xor_u64(v[r], m);
+            const uint64_t other = xor_lane_u64(v[r], m, lane);
             const bool desc_block = (((p & k) == 0) == DESC);
             const bool first = (p & j) == 0;
             const bool keep_max = (first == desc_block);
-            const uint64_t mx = v[r] > other ? v[r] : other;
-            const uint64_t mn = v[r] > other ? other : v[r];
-            v[r] = keep_max ? mx : mn;
+            // keep my key if it is the larger one and I keep the max, or the smaller one and I keep the min
+            v[r] = ((v[r] > other) == keep_max) ? v[r] : other;
         }
     }
 }
@@ -115,10 +136,13 @@ __device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_group
     }
 }
 
-template <typename T, int RK>
+// T: element type of the input and of `scores`; TG: element type of `gates`.  FROM_LOGITS: the input is the raw gate
+// output [num_tokens, 2*nk] (both halves of a token side by side) and the per-half log-softmax is computed here, as
+// torch does it: (v - max) - log(sum(exp(v - max))) in fp32; otherwise the input is [2, num_tokens, nk] scores.
+template <typename T, typename TG, int RK, bool FROM_LOGITS>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
     const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
-    int64_t* __restrict__ indices, T* __restrict__ gates, int norm_topk_prob) {
+    int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob) {
     constexpr int KP = RK * kWave;
     __shared__ uint16_t cand[kMaxCand];
     __shared__ float half_score[kRouterWaves][2][KP];
@@ -146,11 +170,23 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
         if (active) {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const T* row = lp + ((int64_t)h * num_tokens + token) * nk;
+                const T* row = FROM_LOGITS ? lp + (token * 2 + h) * nk : lp + ((int64_t)h * num_tokens + token) * nk;
+                float shift = 0.0f, lse = 0.0f;
+                if (FROM_LOGITS) {
+                    float mx = -INFINITY;
+                    for (int p = lane; p < nk; p += kWave) mx = fmaxf(mx, Elem<T>::to_f32(row[p]));
+                    mx = wave_max(mx);
+                    float se = 0.0f;
+                    for (int p = lane; p < nk; p += kWave) se += expf(Elem<T>::to_f32(row[p]) - mx);
+                    shift = mx;
+                    lse = logf(wave_sum(se));
+                }
                 uint64_t best[RK];
                 topk_groups<RK>(best, lane, half_groups, [&](int g, int r) -> uint64_t {
                     const int p = g * KP + lane * RK + r;
-                    return p < nk ? make_key(Elem<T>::to_f32(row[p]), (uint32_t)p) : 0ull;
+                    if (p >= nk) return 0ull;
+                    const float v = Elem<T>::to_f32(row[p]);
+                    return make_key(FROM_LOGITS ? (v - shift) - lse : v, (uint32_t)p);
                 });
 #pragma unroll
                 for (int r = 0; r < RK; ++r) {
@@ -187,7 +223,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
                     const int64_t o = token * top_k + p;
                     scores[o] = Elem<T>::from_f32(key_score(best[r]));
                     indices[o] = (int64_t)key_index(best[r]);
-                    if (gates != nullptr) gates[o] = Elem<T>::from_f32(norm_topk_prob ? e[r] / total : e[r]);
+                    if (gates != nullptr) gates[o] = Elem<TG>::from_f32(norm_topk_prob ? e[r] / total : e[r]);
                 }
             }
         }
@@ -201,7 +237,7 @@ int count_candidates(int top_k) {
     return n;
 }
 
-template <typename T>
+template <typename T, typename TG, bool FROM_LOGITS>
 int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64_t* indices, void* gates,
                   int norm, hipStream_t stream) {
     const int num_cand = count_candidates(K);
@@ -209,9 +245,9 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
     const int64_t max_blocks = 256 * 8;   // a few resident blocks per CU; the kernel loops over tokens
     const dim3 grid((unsigned)(blocks_needed < max_blocks ? blocks_needed : max_blocks));
     const dim3 block(kRouterWaves * kWave);
-#define FMOE_LAUNCH_ROUTER(R)                                                                                \
-    hipLaunchKernelGGL((router_topk_kernel<T, R>), grid, block, 0, stream, (const T*)lp, T_, nk, K, num_cand, \
-                       (T*)scores, indices, (T*)gates, norm)
+#define FMOE_LAUNCH_ROUTER(R)                                                                                      \
+    hipLaunchKernelGGL((router_topk_kernel<T, TG, R, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, T_, nk, K, \
+                       num_cand, (T*)scores, indices, (TG*)gates, norm)
     if (K <= 64) FMOE_LAUNCH_ROUTER(1);
     else if (K <= 128) FMOE_LAUNCH_ROUTER(2);
     else FMOE_LAUNCH_ROUTER(4);
@@ -221,6 +257,16 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
 }
 
 }  // namespace
+
+int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
+                              int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, hipStream_t stream) {
+    switch (gate_dtype) {
+        case FMOE_F32: return launch_router<float, float, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, stream);
+        case FMOE_BF16: return launch_router<float, bf16_t, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, stream);
+        default: return launch_router<float, f16_t, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, stream);
+    }
+}
+
 }  // namespace fmoe
 
 extern "C" int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
@@ -238,8 +284,8 @@ extern "C" int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int n
     FMOE_REQUIRE(log_probs && scores && indices, FMOE_ERR_NULL_POINTER, "fmoe_router_topk: null tensor pointer");
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FMOE_F32: return launch_router<float>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
-        case FMOE_BF16: return launch_router<bf16_t>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
-        default: return launch_router<f16_t>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+        case FMOE_F32: return launch_router<float, float, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+        case FMOE_BF16: return launch_router<bf16_t, bf16_t, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+        default: return launch_router<f16_t, f16_t, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
     }
 }

@@ -1,0 +1,470 @@
+// Router prologue of the FlashMoE block for gfx950, fused with the product-key top-k:
+//   q = BatchNorm1d(x)  (affine=False; batch statistics in training mode, running statistics otherwise)
+//   logits = q Wr^T     [T, 2*nk]
+//   log-softmax per half, top-k over the pair sums, exp / renormalise   (router_topk_kernel, logits-input mode)
+//
+// Launches:
+//   bn_partial_kernel   per (row block, 512-column strip): shifted sums -> (mean, M2, n) of the block      [training]
+//   bn_finalize_kernel  per column: Chan's parallel combination of the blocks -> mean, 1/sqrt(var+eps);
+//                       running-statistics update (momentum, unbiased variance) and batch counter
+//   router_gate_kernel  MFMA GEMM whose A tile is normalised while it is staged: (x - mean) * rstd is rounded to the
+//                       activation dtype exactly as a stand-alone batch-norm would emit it, then multiplied with the
+//                       gate weights with fp32 accumulation; writes the logits in fp32 (for the routing) and in the
+//                       activation dtype (the tensor the module returns)
+//   router_topk_kernel  (fmoe_router.hip)
+#include <math.h>
+
+#include "fmoe_common.h"
+#include "fmoe_mfma.h"
+
+namespace fmoe {
+namespace {
+
+constexpr int kStatsThreads = 256;
+constexpr int kMaxRowBlocks = 256;
+
+template <typename T> __device__ inline void unpack16(u32x4_t raw, float* v);
+template <> __device__ inline void unpack16<float>(u32x4_t raw, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(raw[i]);
+}
+template <> __device__ inline void unpack16<bf16_t>(u32x4_t raw, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(raw[i] << 16);
+        v[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+    }
+}
+template <> __device__ inline void unpack16<f16_t>(u32x4_t raw, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = raw[i];
+        const f16x2_t p = __builtin_bit_cast(f16x2_t, w);
+        v[2 * i] = (float)p[0];
+        v[2 * i + 1] = (float)p[1];
+    }
+}
+
+// Block (rb, strip): rows [rb*rows_per_block, ...), columns strip*64*V + lane*V .. +V; the 4 waves take rows 4 apart.
+// Sums are taken relative to the block's first row (pivot) so that var = E[d^2] - E[d]^2 does not cancel.
+// partial: [row_blocks][3][H] = (mean, M2, n).
+template <typename T>
+__global__ __launch_bounds__(kStatsThreads) void bn_partial_kernel(const T* __restrict__ x, int64_t num_tokens, int hidden,
+                                                                  int rows_per_block, float* __restrict__ partial) {
+    constexpr int V = Elem<T>::kVec;
+    __shared__ float red[3][2][kWave * V];   // waves 1..3 -> wave 0
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int col = ((int)blockIdx.y * kWave + lane) * V;
+    const bool col_ok = col < hidden;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < num_tokens ? r0 + rows_per_block : num_tokens;
+    float pivot[V], s1[V], s2[V];
+    {
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        if (col_ok) raw = *reinterpret_cast<const u32x4_t*>(x + r0 * hidden + col);
+        unpack16<T>(raw, pivot);
+    }
+#pragma unroll
+    for (int v = 0; v < V; ++v) s1[v] = s2[v] = 0.0f;
+    if (col_ok) {
+        for (int64_t r = r0 + wave; r < r1; r += 4) {
+            float xv[V];
+            unpack16<T>(*reinterpret_cast<const u32x4_t*>(x + r * hidden + col), xv);
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const float d = xv[v] - pivot[v];
+                s1[v] += d;
+                s2[v] = __builtin_fmaf(d, d, s2[v]);
+            }
+        }
+    }
+    // waves 1..3 hand their sums (same pivot) to wave 0 through LDS
+    if (wave > 0) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            red[wave - 1][0][lane * V + v] = s1[v];
+            red[wave - 1][1][lane * V + v] = s2[v];
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                s1[v] += red[w][0][lane * V + v];
+                s2[v] += red[w][1][lane * V + v];
+            }
+    }
+    if (wave == 0 && col_ok) {
+        const float n = (float)(r1 - r0);
+        float* out = partial + (int64_t)blockIdx.x * 3 * hidden;
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            const float m = s1[v] / n;
+            out[col + v] = pivot[v] + m;
+            out[hidden + col + v] = fmaxf(s2[v] - s1[v] * m, 0.0f);
+            out[2 * hidden + col + v] = n;
+        }
+    }
+}
+
+template <typename TS> __device__ inline float load_stat(const void* p, int i) { return Elem<TS>::to_f32(((const TS*)p)[i]); }
+template <typename TS> __device__ inline void store_stat(void* p, int i, float v) { ((TS*)p)[i] = Elem<TS>::from_f32(v); }
+
+// 64 columns per block, 16 waves: wave w takes row-block partials w, w+16, ... (at most kMaxRowBlocks/16 = 16, all
+// loaded before any is used so that one memory round trip covers them).  Two passes: N = sum n_b and
+// mean = sum n_b*mean_b / N, then M2 = sum [M2_b + n_b*(mean_b - mean)^2].
+// training: batch statistics; else the running statistics.  mean_rstd: [2][H] fp32.
+constexpr int kFinalizeWaves = 16;
+template <typename TS>
+__global__ __launch_bounds__(kFinalizeWaves* kWave) void bn_finalize_kernel(
+    const float* __restrict__ partial, int row_blocks, int hidden, int training, float momentum, float eps,
+    void* running_mean, void* running_var, int64_t* num_batches_tracked, float* __restrict__ mean_rstd) {
+    constexpr int PER = kMaxRowBlocks / kFinalizeWaves;
+    __shared__ float red[kFinalizeWaves][2][kWave];
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int h = (int)blockIdx.x * kWave + lane;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && training && num_batches_tracked != nullptr) *num_batches_tracked += 1;
+    const bool h_ok = h < hidden;
+    float mean = 0.0f, m2 = 0.0f, n = 0.0f;
+    if (training) {
+        float mb[PER], m2b[PER], nb[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int b = wave + i * kFinalizeWaves;
+            const bool ok = h_ok && b < row_blocks;
+            const float* p = partial + (int64_t)(ok ? b : 0) * 3 * hidden + (h_ok ? h : 0);
+            mb[i] = ok ? p[0] : 0.0f;
+            m2b[i] = ok ? p[hidden] : 0.0f;
+            nb[i] = ok ? p[2 * hidden] : 0.0f;
+        }
+        float sn = 0.0f, snm = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            sn += nb[i];
+            snm = __builtin_fmaf(nb[i], mb[i], snm);
+        }
+        red[wave][0][lane] = sn;
+        red[wave][1][lane] = snm;
+        __syncthreads();
+        float tn = 0.0f, tnm = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kFinalizeWaves; ++w) {
+            tn += red[w][0][lane];
+            tnm += red[w][1][lane];
+        }
+        n = tn;
+        mean = tnm / fmaxf(tn, 1.0f);
+        __syncthreads();
+        float sm2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const float d = mb[i] - mean;
+            sm2 += __builtin_fmaf(nb[i] * d, d, m2b[i]);
+        }
+        red[wave][0][lane] = sm2;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kFinalizeWaves; ++w) m2 += red[w][0][lane];
+    }
+    if (wave != 0 || !h_ok) return;
+    float var;
+    if (training) {
+        var = m2 / n;                                   // biased: what normalises the batch
+        if (running_mean != nullptr && running_var != nullptr) {
+            const float unbiased = n > 1.0f ? m2 / (n - 1.0f) : var;
+            store_stat<TS>(running_mean, h, (1.0f - momentum) * load_stat<TS>(running_mean, h) + momentum * mean);
+            store_stat<TS>(running_var, h, (1.0f - momentum) * load_stat<TS>(running_var, h) + momentum * unbiased);
+        }
+    } else {
+        mean = load_stat<TS>(running_mean, h);
+        var = load_stat<TS>(running_var, h);
+    }
+    mean_rstd[h] = mean;
+    mean_rstd[hidden + h] = 1.0f / sqrtf(var + eps);
+}
+
+// q = round_T((x - mean) * rstd) for one 16-byte packet
+template <typename T> __device__ inline u32x4_t normalise16(u32x4_t raw, const float* mean, const float* rstd);
+template <> __device__ inline u32x4_t normalise16<bf16_t>(u32x4_t raw, const float* mean, const float* rstd) {
+    float v[8];
+    unpack16<bf16_t>(raw, v);
+    u32x4_t out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bf16x2_t p = {(bf16_t)((v[2 * i] - mean[2 * i]) * rstd[2 * i]), (bf16_t)((v[2 * i + 1] - mean[2 * i + 1]) * rstd[2 * i + 1])};
+        out[i] = __builtin_bit_cast(uint32_t, p);
+    }
+    return out;
+}
+template <> __device__ inline u32x4_t normalise16<f16_t>(u32x4_t raw, const float* mean, const float* rstd) {
+    float v[8];
+    unpack16<f16_t>(raw, v);
+    u32x4_t out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const f16x2_t p = {(f16_t)((v[2 * i] - mean[2 * i]) * rstd[2 * i]), (f16_t)((v[2 * i + 1] - mean[2 * i + 1]) * rstd[2 * i + 1])};
+        out[i] = __builtin_bit_cast(uint32_t, p);
+    }
+    return out;
+}
+
+// logits[M, N] = normalise(x)[M, K] * W[N, K]^T for 16-bit activations: 64x64 tiles (256 of them at T=4096, 2*nk=256),
+// 4 waves of one 32x32 MFMA tile each, register-staged LDS tiles (the A tile is normalised between the global load and
+// the LDS store).  With one such workgroup per CU nothing else hides the global-load latency, so the packets of the
+// next kGatePrefetch k-tiles are kept in flight in registers.
+constexpr int kGatePrefetch = 3;
+constexpr int kGateMaxK = 8192;     // mean / rstd of all k are staged in LDS once: 2 * 4 * K bytes
+
+template <typename T>
+__global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                          const float* __restrict__ mean_rstd, float* __restrict__ logits32,
+                                                          T* __restrict__ logits, int M, int N, int K, int tiles_m,
+                                                          int tiles_n) {
+    using Frag = typename Mfma32<T>::Frag;
+    constexpr int BM = 64, BN = 64, CH = 2;   // CH = 16-byte packets per thread per tile and operand
+    constexpr int D = kGatePrefetch;
+    __shared__ __attribute__((aligned(16))) T As[BM * kTileK];
+    __shared__ __attribute__((aligned(16))) T Bs[BN * kTileK];
+    extern __shared__ __attribute__((aligned(16))) float stats[];   // [2][Kpad]: mean, rstd
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int ch = tid % kTileChunks;          // this thread's packet column inside a k-tile: the same for all its packets
+    const int row0 = tid / kTileChunks;        // rows row0 and row0 + 32
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    const int k_tiles = (K + kTileK - 1) / kTileK;
+    const int kpad = k_tiles * kTileK;
+    for (int i = tid; i < kpad; i += 256) {
+        stats[i] = i < K ? mean_rstd[i] : 0.0f;
+        stats[kpad + i] = i < K ? mean_rstd[K + i] : 0.0f;
+    }
+    u32x4_t ra[D][CH], rb[D][CH];
+
+    auto load_global = [&](int kt, int slot) {
+        const int gk = kt * kTileK + ch * 8;
+        const bool k_ok = kt < k_tiles && gk < K;
+#pragma unroll
+        for (int it = 0; it < CH; ++it) {
+            const int gm = m0 + row0 + it * 32, gn = n0 + row0 + it * 32;
+            ra[slot][it] = (gm < M && k_ok) ? *reinterpret_cast<const u32x4_t*>(x + (int64_t)gm * K + gk) : zero4;
+            rb[slot][it] = (gn < N && k_ok) ? *reinterpret_cast<const u32x4_t*>(w + (int64_t)gn * K + gk) : zero4;
+        }
+    };
+    auto store_lds = [&](int kt, int slot) {
+        const float* mu = stats + kt * kTileK + ch * 8;
+        const float* rs = mu + kpad;
+        float m8[8], r8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            m8[i] = mu[i];
+            r8[i] = rs[i];
+        }
+#pragma unroll
+        for (int it = 0; it < CH; ++it) {
+            *reinterpret_cast<u32x4_t*>(&As[swizzled_offset(row0 + it * 32, ch)]) = normalise16<T>(ra[slot][it], m8, r8);
+            *reinterpret_cast<u32x4_t*>(&Bs[swizzled_offset(row0 + it * 32, ch)]) = rb[slot][it];
+        }
+    };
+    f32x16_t acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    const int frow = lane & 31, fhalf = lane >> 5;
+#pragma unroll
+    for (int d = 0; d < D; ++d) load_global(d, d);
+    __syncthreads();               // stats[] visible
+    // the k loop is unrolled by D so that the register slot of a tile is a compile-time index
+    for (int kt0 = 0; kt0 < k_tiles; kt0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int kt = kt0 + d;
+            if (kt < k_tiles) {
+                store_lds(kt, d);
+                load_global(kt + D, d);        // slot d is free again
+                __syncthreads();
+#pragma unroll
+                for (int ks = 0; ks < kTileK / 16; ++ks) {
+                    const int chunk = ks * 2 + fhalf;
+                    const Frag fa = *reinterpret_cast<const Frag*>(&As[swizzled_offset(wm * 32 + frow, chunk)]);
+                    const Frag fb = *reinterpret_cast<const Frag*>(&Bs[swizzled_offset(wn * 32 + frow, chunk)]);
+                    acc = Mfma32<T>::run(fa, fb, acc);
+                }
+                __syncthreads();
+            }
+        }
+    }
+    const int col = n0 + wn * 32 + frow;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
+        if (row < M && col < N) {
+            logits32[(int64_t)row * N + col] = acc[v];
+            logits[(int64_t)row * N + col] = Elem<T>::from_f32(acc[v]);
+        }
+    }
+}
+
+// fp32 activations (the small parity configuration): plain FMA, 64x64 tile, 4x4 outputs per thread.
+__global__ __launch_bounds__(256) void router_gate_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                              const float* __restrict__ mean_rstd,
+                                                              float* __restrict__ logits32, float* __restrict__ logits,
+                                                              int M, int N, int K) {
+    constexpr int TS = 64, KS = 16;
+    __shared__ float As[KS][TS + 1];
+    __shared__ float Bs[KS][TS + 1];
+    const int m0 = blockIdx.y * TS, n0 = blockIdx.x * TS;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const float* mean = mean_rstd;
+    const float* rstd = mean_rstd + K;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += KS) {
+        for (int q = threadIdx.x; q < TS * KS; q += 256) {
+            const int r = q / KS, kk = q % KS, gk = k0 + kk;
+            As[kk][r] = (m0 + r < M && gk < K) ? (x[(int64_t)(m0 + r) * K + gk] - mean[gk]) * rstd[gk] : 0.0f;
+            Bs[kk][r] = (n0 + r < N && gk < K) ? w[(int64_t)(n0 + r) * K + gk] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                a[i] = As[kk][ty * 4 + i];
+                b[i] = Bs[kk][tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = m0 + ty * 4 + i, col = n0 + tx * 4 + j;
+            if (row < M && col < N) {
+                logits32[(int64_t)row * N + col] = acc[i][j];
+                logits[(int64_t)row * N + col] = acc[i][j];
+            }
+        }
+}
+
+struct ProloguePlan {
+    int row_blocks, rows_per_block;
+    size_t off_partial, off_mean_rstd, bytes;
+};
+
+ProloguePlan plan_prologue(int64_t T_, int H, int nk) {
+    ProloguePlan p;
+    int64_t rb = (T_ + 31) / 32;
+    p.row_blocks = (int)(rb < 1 ? 1 : (rb > kMaxRowBlocks ? kMaxRowBlocks : rb));
+    p.rows_per_block = (int)((T_ + p.row_blocks - 1) / p.row_blocks);
+    p.row_blocks = (int)((T_ + p.rows_per_block - 1) / p.rows_per_block);
+    p.off_partial = 0;
+    p.off_mean_rstd = round_up((size_t)kMaxRowBlocks * 3 * (size_t)H * 4, 256);
+    (void)nk;
+    p.bytes = round_up(p.off_mean_rstd + 2 * (size_t)H * 4, 256);
+    return p;
+}
+
+template <typename T>
+void launch_stats(const void* x, int64_t T_, int H, const ProloguePlan& p, float* partial, hipStream_t stream) {
+    constexpr int V = Elem<T>::kVec;
+    const int strips = (H + kWave * V - 1) / (kWave * V);
+    hipLaunchKernelGGL((bn_partial_kernel<T>), dim3((unsigned)p.row_blocks, (unsigned)strips), dim3(kStatsThreads), 0, stream,
+                       (const T*)x, T_, H, p.rows_per_block, partial);
+}
+
+template <typename TS>
+void launch_finalize(const float* partial, const ProloguePlan& p, int H, int training, float momentum, float eps,
+                     void* rm, void* rv, int64_t* nbt, float* mean_rstd, hipStream_t stream) {
+    hipLaunchKernelGGL((bn_finalize_kernel<TS>), dim3((unsigned)((H + kWave - 1) / kWave)), dim3(kFinalizeWaves * kWave), 0, stream, partial,
+                       p.row_blocks, H, training, momentum, eps, rm, rv, nbt, mean_rstd);
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" size_t fmoe_router_workspace_bytes(int64_t num_tokens, int hidden, int num_keys) {
+    if (num_tokens <= 0 || hidden <= 0 || num_keys <= 0) return 0;
+    return fmoe::plan_prologue(num_tokens, hidden, num_keys).bytes;
+}
+
+extern "C" int fmoe_router_forward(const void* x, const void* gate_w, void* running_mean, void* running_var,
+                                   int64_t* num_batches_tracked, int stats_dtype, int training, float momentum,
+                                   float eps, int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype,
+                                   int norm_topk_prob, void* router_logits, float* logits_fp32, float* scores,
+                                   int64_t* indices, void* gates, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype) && dtype_ok(stats_dtype), FMOE_ERR_BAD_DTYPE,
+                 "fmoe_router_forward: unknown dtype %d / statistics dtype %d", dtype, stats_dtype);
+    FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_keys > 0, FMOE_ERR_BAD_SHAPE,
+                 "fmoe_router_forward: bad shape T=%lld H=%d nk=%d", (long long)num_tokens, hidden, num_keys);
+    FMOE_REQUIRE(top_k >= 0 && top_k <= num_keys, FMOE_ERR_TOPK_RANGE,
+                 "num_experts_per_tok should be in [0, %d], but got %d", num_keys, top_k);
+    FMOE_REQUIRE(dtype == FMOE_F32 || hidden <= kGateMaxK, FMOE_ERR_UNSUPPORTED,
+                 "fmoe_router_forward: hidden=%d > %d for 16-bit activations", hidden, kGateMaxK);
+    FMOE_REQUIRE(num_keys <= 32767 && top_k <= 256 && num_tokens < (1ll << 31), FMOE_ERR_UNSUPPORTED,
+                 "fmoe_router_forward: nk=%d top_k=%d T=%lld beyond what the kernels are built for", num_keys, top_k,
+                 (long long)num_tokens);
+    if (num_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(!(training && num_tokens == 1), FMOE_ERR_BAD_SHAPE,
+                 "Expected more than 1 value per channel when training, got input size [1, %d]", hidden);
+    FMOE_REQUIRE(x && gate_w && router_logits && logits_fp32 && workspace, FMOE_ERR_NULL_POINTER,
+                 "fmoe_router_forward: null tensor pointer");
+    FMOE_REQUIRE(top_k == 0 || (scores && indices), FMOE_ERR_NULL_POINTER, "fmoe_router_forward: null scores/indices");
+    FMOE_REQUIRE(training || (running_mean && running_var), FMOE_ERR_NULL_POINTER,
+                 "fmoe_router_forward: evaluation mode needs running statistics");
+    const int vec = (int)(16 / dtype_size(dtype));
+    FMOE_REQUIRE(hidden % vec == 0 && aligned16(x) && aligned16(gate_w), FMOE_ERR_ALIGNMENT,
+                 "fmoe_router_forward: hidden=%d must be a multiple of %d and tensors 16-byte aligned", hidden, vec);
+    const ProloguePlan p = plan_prologue(num_tokens, hidden, num_keys);
+    FMOE_REQUIRE(workspace_bytes >= p.bytes && aligned16(workspace), FMOE_ERR_WORKSPACE,
+                 "fmoe_router_forward: workspace of %zu bytes needed, %zu given", p.bytes, workspace_bytes);
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    float* partial = (float*)(ws + p.off_partial);
+    float* mean_rstd = (float*)(ws + p.off_mean_rstd);
+    float* logits32 = logits_fp32;
+
+    if (training) {
+        switch (dtype) {
+            case FMOE_F32: launch_stats<float>(x, num_tokens, hidden, p, partial, s); break;
+            case FMOE_BF16: launch_stats<bf16_t>(x, num_tokens, hidden, p, partial, s); break;
+            default: launch_stats<f16_t>(x, num_tokens, hidden, p, partial, s); break;
+        }
+        FMOE_CHECK_LAUNCH("fmoe_router_forward(batch statistics)");
+    }
+    switch (stats_dtype) {
+        case FMOE_F32: launch_finalize<float>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+        case FMOE_BF16: launch_finalize<bf16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+        default: launch_finalize<f16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+    }
+    FMOE_CHECK_LAUNCH("fmoe_router_forward(finalize)");
+
+    const int M = (int)num_tokens, N = 2 * num_keys;
+    if (dtype == FMOE_F32) {
+        hipLaunchKernelGGL(router_gate_f32_kernel, dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, s, (const float*)x,
+                           (const float*)gate_w, (const float*)mean_rstd, logits32, (float*)router_logits, M, N, hidden);
+    } else {
+        const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
+        const size_t stats_bytes = (size_t)((hidden + kTileK - 1) / kTileK) * kTileK * 2 * sizeof(float);
+        if (dtype == FMOE_BF16)
+            hipLaunchKernelGGL((router_gate_kernel<bf16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
+                               (const bf16_t*)x, (const bf16_t*)gate_w, (const float*)mean_rstd, logits32,
+                               (bf16_t*)router_logits, M, N, hidden, tiles_m, tiles_n);
+        else
+            hipLaunchKernelGGL((router_gate_kernel<f16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
+                               (const f16_t*)x, (const f16_t*)gate_w, (const float*)mean_rstd, logits32,
+                               (f16_t*)router_logits, M, N, hidden, tiles_m, tiles_n);
+    }
+    FMOE_CHECK_LAUNCH("fmoe_router_forward(gate)");
+    if (top_k == 0) return FMOE_OK;
+    return launch_router_from_logits(logits32, num_tokens, num_keys, top_k, scores, indices, gates, dtype, norm_topk_prob, s);
+}

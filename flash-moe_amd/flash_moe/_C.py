@@ -30,6 +30,9 @@ SIGNATURES = {
     "fmoe_abi_version": (_int, []),
     "fmoe_last_error": (ctypes.c_char_p, []),
     "fmoe_router_topk": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp, _vp, _int, _vp]),
+    "fmoe_router_workspace_bytes": (_sz, [_i64, _int, _int]),
+    "fmoe_router_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int,
+                                   _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_expert_workspace_bytes": (_sz, [_i64, _int, _i64, _int, _int]),
     "fmoe_expert_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_expert_forward_algo": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _int, _vp]),

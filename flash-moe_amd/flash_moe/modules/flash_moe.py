@@ -5,12 +5,11 @@ six arguments (flash_moe/modules/flash_moe.py:12-27), ``FlashMoE`` owns paramete
 the same ``state_dict`` names (:43-53) and ``forward`` returns the same ``(hidden_states, router_logits)``
 pair (:55-105).
 
-Stages of ``forward`` and where each runs:
-  batch-norm + router gate     torch (statistics and a [T,H]x[H,2nk] product)
-  log-softmax                  torch, always in fp32
-  product-key top-k + gates    ``fmoe_router_topk``   (HIP)
-  routed experts               ``fmoe_expert_forward`` (HIP)
-  shared SwiGLU MLP + add      ``fmoe_mlp_forward``    (HIP; the add is the second GEMM's epilogue)
+Stages of ``forward``, all HIP:
+  batch-norm, router gate, log-softmax, product-key top-k, gates    ``fmoe_router_forward``
+  routed experts                                                    ``fmoe_expert_forward``
+  shared SwiGLU MLP + add                                           ``fmoe_mlp_forward`` (the add is the second
+                                                                    GEMM's epilogue)
 
 Routing is evaluated in fp32 whatever the module dtype: the normalised activations are rounded to the
 module dtype exactly as the reference does, but their product with the router gate, the log-softmax
@@ -29,7 +28,7 @@ import torch.nn.functional as F
 
 from flash_moe.ops.hip.flash_expert import expert_forward
 from flash_moe.ops.hip.flash_mlp import mlp_forward
-from flash_moe.ops.hip.flash_router import router_topk_gates
+from flash_moe.ops.hip.flash_router import router_forward
 
 _SILU_NAMES = ("silu", "swish")
 
@@ -75,32 +74,20 @@ class FlashMoE(nn.Module):
         self.down_embed = nn.Embedding(E, H)
         self.up_embed = nn.Embedding(E, H)
 
-    def router_log_probs(self, tokens: torch.Tensor):
-        """[T, H] -> (logits [T, 2*nk] fp32, log-probabilities [2, T, nk] fp32).  In training mode this
-        updates the batch-norm running statistics, like any call of the module."""
-        T = tokens.shape[0]
-        q = self.router_norm(tokens)
-        logits32 = F.linear(q.float(), self.router_gate.weight.float())
-        log_probs = F.log_softmax(logits32.view(T, 2, self.num_keys), dim=-1).transpose(0, 1)
-        return logits32, log_probs
-
-    def route(self, tokens: torch.Tensor):
-        """[T, H] -> (router_logits [2, T, nk] in the module dtype, scores, indices int64, gates)."""
-        T = tokens.shape[0]
-        logits32, log_probs = self.router_log_probs(tokens)
-        scores, indices, gates = router_topk_gates(
-            log_probs, self.num_keys, self.top_k, with_gates=True, norm_topk_prob=self.norm_topk_prob
-        )
-        router_logits = logits32.to(tokens.dtype).view(T, 2, self.num_keys).transpose(0, 1)
-        return router_logits, scores, indices, gates
+    def route(self, tokens: torch.Tensor, return_logits32: bool = False):
+        """[T, H] -> (router_logits [2, T, nk] in the module dtype, scores fp32, indices int64, gates); with
+        ``return_logits32`` also the fp32 gate output [T, 2*nk] the routing was computed from.  Like any forward call
+        this updates the batch-norm running statistics in training mode."""
+        out = router_forward(tokens, self.router_gate.weight, self.router_norm, self.num_keys, self.top_k,
+                             self.norm_topk_prob, return_logits32)
+        router_logits = out[0].view(tokens.shape[0], 2, self.num_keys).transpose(0, 1)
+        return (router_logits,) + tuple(out[1:])
 
     def forward(self, hidden_states: torch.Tensor, **kwargs):
         bsz, seq_len, _ = hidden_states.shape
         tokens = hidden_states.view(-1, self.hidden_size)
         router_logits, _, indices, gates = self.route(tokens)
-        experts_states = expert_forward(
-            tokens, self.down_embed.weight, self.up_embed.weight, indices, gates.to(tokens.dtype)
-        )
+        experts_states = expert_forward(tokens, self.down_embed.weight, self.up_embed.weight, indices, gates)
         out = mlp_forward(
             tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, residual=experts_states
         )

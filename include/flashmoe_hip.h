@@ -67,6 +67,34 @@ int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, in
                      void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Router of the block, from the block's input to gates: everything FlashMoE.forward does before it calls the
+ * expert op (flash_moe/modules/flash_moe.py:62-85): BatchNorm1d(affine=False) -> router_gate (Linear, no bias) ->
+ * per-half log-softmax -> triton_flash_router_func -> exp -> optional renormalisation.
+ *
+ *   x              [T, H]        dtype   block input
+ *   gate_w         [2*nk, H]     dtype   router_gate.weight (rows [0,nk) score half 0, rows [nk,2nk) half 1)
+ *   running_mean / running_var [H], num_batches_tracked [1] int64: router_norm's buffers, element type stats_dtype.
+ *                  training != 0: batch statistics normalise x and the buffers are updated as nn.BatchNorm1d does
+ *                  (momentum, unbiased variance; the counter is incremented); they may be NULL to skip the update.
+ *                  training == 0: the running statistics normalise x.
+ *   router_logits  [T, 2*nk]     dtype   out: the gate output the module returns (as a [2,T,nk] view)
+ *   logits_fp32    [T, 2*nk]     fp32    out: the same before rounding; the routing is computed from these
+ *   scores         [T, top_k]    fp32    out: log-probability sums, descending
+ *   indices        [T, top_k]    int64   out: expert ids i*nk + j
+ *   gates          [T, top_k]    dtype   out: routing weights (NULL to skip)
+ * The normalised activations are rounded to dtype as a stand-alone batch-norm emits them; the product with gate_w,
+ * the log-softmax and the pair sums are fp32.  With T == 1 in training mode the call is rejected like
+ * nn.BatchNorm1d rejects it.  workspace: fmoe_router_workspace_bytes() bytes, 256-byte aligned.
+ */
+size_t fmoe_router_workspace_bytes(int64_t num_tokens, int hidden, int num_keys);
+
+int fmoe_router_forward(const void* x, const void* gate_w, void* running_mean, void* running_var,
+                        int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
+                        int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
+                        void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Routed experts.
  * Replaces triton_flash_expert_func / FlashExpertFunc.forward / _flash_expert_forward and its host-side
  * preprocessing (flash_moe/ops/triton/flash_expert.py:831-836, 748-796, 580-651, 528-577; contract

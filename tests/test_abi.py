@@ -63,6 +63,25 @@ def test_router_argument_checks():
     assert lib.fmoe_last_error() == b""
 
 
+def test_fused_router_argument_checks():
+    lib = _C.lib()
+    keep, a = _buf()
+    f = lib.fmoe_router_forward
+    need = lib.fmoe_router_workspace_bytes(64, 128, 16)
+    assert need > 0 and need % 256 == 0
+    ok_args = dict(x=a, w=a, rm=a, rv=a, nbt=a)
+    call = lambda **kw: f(kw.get("x", a), a, a, a, a, _C.F32, kw.get("training", 1), 0.1, 1e-5, kw.get("T", 64), 128, 16,
+                          kw.get("K", 4), kw.get("dtype", _C.BF16), 0, a, a, a, a, a, kw.get("ws", a), kw.get("wsb", need), None)
+    assert call(K=17) == -3                       # top_k > num_keys
+    assert call(dtype=9) == -4
+    assert call(T=-1) == -2
+    assert call(T=1) == -2                        # one token in training mode, as nn.BatchNorm1d
+    assert b"more than 1 value per channel" in lib.fmoe_last_error()
+    assert call(x=None) == -1
+    assert call(wsb=need - 1) == -7
+    assert call(T=0) == 0
+
+
 def test_expert_argument_checks():
     lib = _C.lib()
     keep, a = _buf()

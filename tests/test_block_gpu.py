@@ -41,20 +41,19 @@ def stagewise_check(m, w, x, K, norm, dtype):
     # stage by stage on the HIP path's intermediates
     m.router_norm.reset_running_stats()
     tokens = x.cuda().view(-1, H)
-    _, lp = m.router_log_probs(tokens)
-    m.router_norm.reset_running_stats()
-    _, scores, indices, gates = m.route(tokens)
-    idx_cpu, gates_cpu = indices.cpu(), gates.cpu()
-    # router stage on identical input: the oracle's top-k of the HIP path's own fp32 log-probabilities
-    lp_cpu = lp.contiguous().cpu()
+    _, scores, indices, gates, logits32 = m.route(tokens, return_logits32=True)
+    idx_cpu, gates_cpu = indices.cpu(), gates.float().cpu()
+    # router stage on identical input: the oracle's log-softmax and top-k of the HIP path's own fp32 gate output
+    lp_cpu = torch.log_softmax(logits32.cpu().view(T, 2, nk), dim=-1).transpose(0, 1).contiguous()
     Kx = K + 1
     o_s = torch.cat([orc.router_topk(lp_cpu[:, lo:lo + 256].contiguous(), nk, Kx)[0] for lo in range(0, T, 256)])
     o_i = torch.cat([orc.router_topk(lp_cpu[:, lo:lo + 256].contiguous(), nk, Kx)[1] for lo in range(0, T, 256)])
-    assert torch.equal(scores.cpu(), o_s[:, :K])
+    torch.testing.assert_close(scores.cpu(), o_s[:, :K], rtol=0, atol=2e-6)     # log-softmax differs in the last ulp
     set_equal = (idx_cpu.sort(-1).values == o_i[:, :K].sort(-1).values).all(-1)
-    tie_at_cut = (o_s[:, K - 1] - o_s[:, K]).abs() < 1e-6
+    tie_at_cut = (o_s[:, K - 1] - o_s[:, K]).abs() < 2e-6
     assert (set_equal | tie_at_cut).all()
-    torch.testing.assert_close(gates_cpu, orc.routing_weights(o_s[:, :K], norm), rtol=1e-5, atol=1e-10)
+    g_tol = {torch.float32: 1e-5, torch.bfloat16: 8e-3, torch.float16: 1e-3}[dtype]
+    torch.testing.assert_close(gates_cpu, orc.routing_weights(o_s[:, :K], norm), rtol=g_tol, atol=1e-10)
     # end to end the selection is chaotic: a one-ulp difference in a 16-bit batch-norm output moves a logit
     # by ~1e-4 and can swap the experts around the cut, so only the overlap with the oracle's sets is bounded
     hit = torch.tensor([len(set(a.tolist()) & set(b.tolist())) for a, b in zip(idx_cpu, ref["indices"])]).float()
@@ -63,9 +62,9 @@ def stagewise_check(m, w, x, K, norm, dtype):
     # experts: oracle on the HIP path's own indices and gates
     from flash_moe.ops.hip.flash_expert import expert_forward
 
-    e_hip = expert_forward(tokens, m.down_embed.weight, m.up_embed.weight, indices, gates.to(dtype)).cpu()
+    e_hip = expert_forward(tokens, m.down_embed.weight, m.up_embed.weight, indices, gates).cpu()
     e_ref = orc.expert_forward(x.view(-1, H).double(), w.down_embed.double(), w.up_embed.double(), idx_cpu,
-                               gates_cpu.to(dtype).double(), token_chunk=256)
+                               gates.cpu().double(), token_chunk=256)
     fro = rel_fro(e_hip, e_ref)
     assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 1e-3}[dtype], f"experts: {fro:.3e}"
     # block output against a float64 evaluation of MLP + experts on the HIP path's own routing: only the
@@ -113,7 +112,7 @@ def test_block_c4_full_size_properties():
     tokens = x.view(-1, 1024)
     _, _, indices, gates = m.route(tokens)
     parts = flash_mlp_func(tokens, m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight).float() + expert_forward(
-        tokens, m.down_embed.weight, m.up_embed.weight, indices, gates.to(dtype)).float()
+        tokens, m.down_embed.weight, m.up_embed.weight, indices, gates).float()
     assert rel_fro(y1.view(-1, 1024), parts) < 6e-3
     # gates are probabilities p_x * p_y of distinct experts
     assert (gates > 0).all() and (gates.sum(-1) <= 1 + 1e-3).all()

@@ -129,3 +129,97 @@ def test_router_noncontiguous_input_and_empty():
     assert s0.shape == (T, 0) and i0.shape == (T, 0)
     se, ie = flash_router_func(torch.empty(2, 0, nk, device="cuda"), nk, K)
     assert se.shape == (0, K)
+
+
+# ------------------------------------------------------------------------------------------------
+# the block's fused routing stage (batch-norm -> gate -> log-softmax -> top-k -> gates)
+# ------------------------------------------------------------------------------------------------
+def _fused(x, wr, nk, K, norm_flag, dtype, training=True, rm=None, rv=None):
+    from flash_moe.ops.hip.flash_router import router_forward
+
+    H = x.shape[1]
+    bn = torch.nn.BatchNorm1d(H, affine=False)
+    if rm is not None:
+        bn.running_mean.copy_(rm); bn.running_var.copy_(rv)
+    bn = bn.to(device="cuda", dtype=dtype)
+    bn.train(training)
+    out = router_forward(x.to(dtype).cuda(), wr.to(dtype).cuda(), bn, nk, K, norm_flag, return_logits32=True)
+    return out, bn
+
+
+@pytest.mark.parametrize("T,H,nk,K", [(512, 256, 32, 16), (1000, 1024, 128, 64), (130, 72, 100, 37), (64, 2048, 512, 128)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_fused_router_matches_oracle_prologue(T, H, nk, K, dtype):
+    g = torch.Generator().manual_seed(T + nk)
+    x = (torch.randn(T, H, generator=g) * 1.7 + 0.3).to(dtype)
+    wr = (torch.randn(2 * nk, H, generator=g) * 0.02).to(dtype)
+    (logits, scores, indices, gates, logits32), bn = _fused(x.float(), wr.float(), nk, K, False, dtype)
+    assert logits.shape == (T, 2 * nk) and logits.dtype == dtype and logits32.dtype == torch.float32
+    # oracle: batch-norm as torch runs it in this dtype, the rest in fp32 on those values
+    rm, rv = torch.zeros(H, dtype=dtype), torch.ones(H, dtype=dtype)
+    q = torch.nn.functional.batch_norm(x, rm, rv, None, None, True, 0.1, 1e-5)
+    ref32 = torch.nn.functional.linear(q.float(), wr.float())
+    tol = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}[dtype]
+    torch.testing.assert_close(logits.float().cpu(), ref32.to(dtype).float(), rtol=tol, atol=tol)
+    # fp32 logits against the CPU oracle: its 16-bit batch-norm keeps mean and 1/std in 16 bits, so the normalised
+    # activations differ by a 16-bit rounding
+    fro = ((logits32.cpu() - ref32).norm() / ref32.norm()).item()
+    assert fro < {torch.float32: 1e-5, torch.bfloat16: 6e-3, torch.float16: 1e-3}[dtype], fro
+    # ... and against torch's batch-norm on this device (fp32 statistics, the routine the reference module calls):
+    # only a rare one-ulp difference of a normalised activation remains
+    q_dev = torch.nn.functional.batch_norm(x.cuda(), None, None, None, None, True, 0.1, 1e-5)
+    ref_dev = torch.nn.functional.linear(q_dev.float().cpu(), wr.float())
+    fro = ((logits32.cpu() - ref_dev).norm() / ref_dev.norm()).item()
+    assert fro < {torch.float32: 1e-5, torch.bfloat16: 5e-4, torch.float16: 1e-4}[dtype], fro
+    # running statistics follow nn.BatchNorm1d (momentum 0.1, unbiased variance), counter incremented
+    torch.testing.assert_close(bn.running_mean.float().cpu(), rm.float(), rtol=2e-2, atol=2e-3)
+    torch.testing.assert_close(bn.running_var.float().cpu(), rv.float(), rtol=2e-2, atol=2e-3)
+    assert int(bn.num_batches_tracked) == 1
+    # routing stage on identical input: oracle log-softmax + top-k of the fp32 logits the kernel produced
+    lp = torch.log_softmax(logits32.cpu().view(T, 2, nk), -1).transpose(0, 1).contiguous()
+    o_s, o_i = oracle_topk_chunked(lp, nk, min(K + 1, nk * nk))
+    torch.testing.assert_close(scores.cpu(), o_s[:, :K], rtol=0, atol=2e-6)
+    same = (indices.cpu().sort(-1).values == o_i[:, :K].sort(-1).values).all(-1)
+    tie = (o_s[:, K - 1] - o_s[:, K]).abs() < 2e-6 if o_s.shape[1] > K else torch.zeros(T, dtype=torch.bool)
+    assert (same | tie).all()
+    g_tol = {torch.float32: 1e-5, torch.bfloat16: 8e-3, torch.float16: 1e-3}[dtype]
+    torch.testing.assert_close(gates.float().cpu(), orc.routing_weights(o_s[:, :K], False), rtol=g_tol, atol=1e-10)
+
+
+def test_fused_router_eval_mode_and_normalised_gates():
+    T, H, nk, K = 300, 128, 64, 32
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, H, generator=g) * 2 + 1
+    wr = torch.randn(2 * nk, H, generator=g) * 0.05
+    rm, rv = torch.randn(H, generator=g), torch.rand(H, generator=g) + 0.5
+    (logits, scores, indices, gates, logits32), bn = _fused(x, wr, nk, K, True, torch.float32, training=False, rm=rm, rv=rv)
+    ref_logits, ref_lp = orc.router_prologue(x, wr, nk, rm.clone(), rv.clone(), training=False)
+    torch.testing.assert_close(logits.cpu().view(T, 2, nk).transpose(0, 1), ref_logits, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(bn.running_mean.cpu(), rm) and int(bn.num_batches_tracked) == 0   # untouched in eval mode
+    torch.testing.assert_close(gates.sum(-1).cpu(), torch.ones(T), rtol=1e-5, atol=1e-5)
+    o_s, o_i = orc.router_topk(ref_lp, nk, K)
+    overlap = sum(len(set(a.tolist()) & set(b.tolist())) for a, b in zip(indices.cpu(), o_i)) / o_i.numel()
+    assert overlap > 0.999
+
+
+def test_fused_router_statistics_are_stable_for_offset_data():
+    # a large common offset must not cancel in the variance
+    T, H, nk, K = 2048, 64, 16, 4
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(T, H, generator=g) * 0.01 + 100.0
+    wr = torch.randn(2 * nk, H, generator=g)
+    (logits, *_), bn = _fused(x, wr, nk, K, False, torch.float32)
+    ref_logits, _ = orc.router_prologue(x.double(), wr.double(), nk)
+    err = (logits.cpu().double().view(T, 2, nk).transpose(0, 1) - ref_logits).abs().max().item()
+    assert err < 2e-2 * ref_logits.abs().max().item(), err
+
+
+def test_fused_router_rejects_single_token_in_training():
+    from flash_moe.ops.hip.flash_router import router_forward
+
+    bn = torch.nn.BatchNorm1d(64, affine=False).cuda()
+    with pytest.raises(ValueError, match="more than 1 value per channel"):
+        router_forward(torch.randn(1, 64, device="cuda"), torch.randn(16, 64, device="cuda"), bn, 8, 4)
+    bn.eval()
+    out = router_forward(torch.randn(1, 64, device="cuda"), torch.randn(16, 64, device="cuda"), bn, 8, 4)
+    assert out[2].shape == (1, 4)
