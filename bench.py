@@ -249,6 +249,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-c3", action="store_true")
+    ap.add_argument("--only-c3", action="store_true", help="run only the routed-expert kernel on its own shape (for profiling)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a 256 MiB device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (the forward path is single-GPU; "
@@ -265,6 +268,19 @@ def main():
     _C.lib()   # fail loudly here if the HIP library is missing
     dtype = torch.bfloat16
     torch.cuda.set_device(0)
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.only_c3:
+        res = bench_expert_c3(dtype, max(10, min(50, args.steps)))
+        log("expert C3:", res)
+        print(json.dumps({"metric": "expert kernel HBM GB/s", "value": res["achieved_GBps"], "unit": "GB/s", "n_gpus": 1,
+                          "steps": args.steps, "warmup": args.warmup, "expert_c3": res}), flush=True)
+        return
     m, x = synthetic_block(C4, dtype, "cuda:0")
     T = C4["batch"] * C4["seq"]
 
