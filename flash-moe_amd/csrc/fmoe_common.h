@@ -35,9 +35,27 @@ void clear_error();
     } while (0)
 
 // Top-k of the router taking raw fp32 gate outputs [T, 2*nk] (log-softmax per half is done inside); defined in
-// fmoe_router.hip, used by the fused router entry point.  gates has element type `gate_dtype`.
+// fmoe_router.hip, used by the fused router entry point.  gates has element type `gate_dtype`.  When `row_offsets`
+// is given, the byte offset id*row_bytes of each selected expert's table row is written next to its id.
 int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
-                              int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, hipStream_t stream);
+                              int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, uint32_t* row_offsets,
+                              uint32_t row_bytes, hipStream_t stream);
+
+// The fused router (fmoe_router_forward) with the optional row-offset output; defined in fmoe_router_prologue.hip.
+int router_forward_impl(const void* x, const void* gate_w, void* running_mean, void* running_var,
+                        int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
+                        int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
+                        void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
+                        uint32_t* row_offsets, uint32_t row_bytes, void* workspace, size_t workspace_bytes,
+                        hipStream_t stream);
+
+// Column-slice schedule of the routed experts on row offsets that are already in place at the start of `workspace`
+// (the layout fmoe_expert_workspace_bytes describes); defined in fmoe_expert.hip.
+bool expert_slices_usable(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
+uint32_t* expert_workspace_offsets(void* workspace);
+int expert_slices_prepared(const void* x, const void* down, const void* up, const void* gates, int64_t num_tokens,
+                           int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
+                           hipStream_t stream);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline size_t dtype_size(int dtype) { return dtype == FMOE_F32 ? 4 : 2; }

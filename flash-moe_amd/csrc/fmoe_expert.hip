@@ -414,31 +414,41 @@ SlicePlan plan_slices(int64_t T_, int H, int K, size_t elt) {
     return p;
 }
 
+// Scores, gate and states launches on row offsets that already sit at the start of the workspace.
 template <typename T>
-int launch_expert_slices(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
-                         int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+int launch_expert_slices_prepared(const void* x, const void* down, const void* up, const void* gates, int64_t T_, int H,
+                                  int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
     const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
     char* ws = (char*)workspace;
-    uint32_t* off32 = (uint32_t*)(ws + p.off_idx32);
-    const uint32_t row_bytes = (uint32_t)(H * sizeof(T));
-    const uint32_t table_bytes = (uint32_t)(E * (int64_t)row_bytes);
+    const uint32_t* off32 = (const uint32_t*)(ws + p.off_idx32);
+    const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
     float* a = (float*)(ws + p.off_a);
     float* spart = (float*)(ws + p.off_spart);
     const int64_t pairs = T_ * K;
     const unsigned flat_grid = (unsigned)((pairs + 255) / 256);
-    hipLaunchKernelGGL(expert_prepare_kernel, dim3(flat_grid), dim3(256), 0, stream, indices, off32, pairs, E, row_bytes);
-    FMOE_CHECK_LAUNCH("fmoe_expert_forward(prepare)");
     hipLaunchKernelGGL((expert_scores_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const T*)x, (const T*)down,
-                       table_bytes, (const uint32_t*)off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+                       table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(scores)");
     hipLaunchKernelGGL((expert_gate_kernel<T>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
-                       (const T*)gates, (const uint32_t*)off32, a, pairs, p.num_slices);
+                       (const T*)gates, off32, a, pairs, p.num_slices);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(gate)");
     hipLaunchKernelGGL((expert_states_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
-                       (const T*)up, table_bytes, (const uint32_t*)off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
+                       (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
                        p.tokens_per_block);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(states)");
     return FMOE_OK;
+}
+
+template <typename T>
+int launch_expert_slices(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
+                         int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+    const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
+    uint32_t* off32 = (uint32_t*)((char*)workspace + p.off_idx32);
+    const int64_t pairs = T_ * K;
+    hipLaunchKernelGGL(expert_prepare_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, indices, off32,
+                       pairs, E, (uint32_t)(H * sizeof(T)));
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(prepare)");
+    return launch_expert_slices_prepared<T>(x, down, up, gates, T_, H, E, K, out, workspace, stream);
 }
 
 // A 128-byte slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic;
@@ -449,6 +459,23 @@ bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) &&
 bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
 
 }  // namespace
+
+bool expert_slices_usable(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
+    return top_k > 0 && slices_pay(num_tokens, num_experts, top_k) && slices_possible(num_experts, hidden, dtype_size(dtype));
+}
+
+uint32_t* expert_workspace_offsets(void* workspace) { return (uint32_t*)workspace; }   // SlicePlan::off_idx32 == 0
+
+int expert_slices_prepared(const void* x, const void* down, const void* up, const void* gates, int64_t num_tokens,
+                           int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
+                           hipStream_t stream) {
+    switch (dtype) {
+        case FMOE_F32: return launch_expert_slices_prepared<float>(x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+        case FMOE_BF16: return launch_expert_slices_prepared<bf16_t>(x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+        default: return launch_expert_slices_prepared<f16_t>(x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+    }
+}
+
 }  // namespace fmoe
 
 extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {

@@ -208,12 +208,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 
     __shared__ __attribute__((aligned(1024))) T lds[NSTAGE * STAGE];
 
-    int tm, tn;
-    tile_of_block(tiles_m, tiles_n, tm, tn);
-    const int m0 = tm * BM, n0 = tn * BN_OUT;
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int num_tiles = tiles_m * tiles_n;
 
     // DMA: the lane's LDS position is row (round*ROWS_PER_IT + wave*RPI + lrow), physical chunk lp; it holds the
     // logical chunk lp ^ key(row), key(row) = (row >> ROW_SHIFT) & (CPR-1).  ROWS_PER_IT is a multiple of 16, so the
@@ -221,10 +219,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     const int lrow = lane / CPR, lp = lane % CPR;
     const int key_dma = ((wave * RPI + lrow) >> ROW_SHIFT) & (CPR - 1);
     const int lane_off = lrow * K + ((lp ^ key_dma) << 3);
-    const T* a_src = A + (int64_t)(m0 + wave * RPI) * K + lane_off;
-    const T* b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K + lane_off;
-    const T* b_src1 = (EPI == kEpiSwiGLU) ? B1 + (int64_t)(n0 + wave * RPI) * K + lane_off : nullptr;
-
+    const T *a_src, *b_src0, *b_src1 = nullptr;
+    int m0, n0;
+    // The workgroup is persistent: it takes tiles t, t + gridDim.x, ...  Each XCD (workgroup id mod 8) gets a contiguous
+    // run of the tile order, walked 8 tile-rows at a time so that a compact patch shares A and B tiles in the XCD's L2.
+    auto set_tile = [&](int t) {
+        if ((num_tiles & 7) == 0) t = (t & 7) * (num_tiles >> 3) + (t >> 3);
+        constexpr int GM = 8;
+        const int width = GM * tiles_n, group = t / width, first_m = group * GM;
+        const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+        m0 = (first_m + (t % width) % gsz) * BM;
+        n0 = ((t % width) / gsz) * BN_OUT;
+        a_src = A + (int64_t)(m0 + wave * RPI) * K + lane_off;
+        b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K + lane_off;
+        if (EPI == kEpiSwiGLU) b_src1 = B1 + (int64_t)(n0 + wave * RPI) * K + lane_off;
+    };
     auto issue = [&](int kt, T* stage) {
         const int k0 = kt * BKT;
 #pragma unroll
@@ -242,14 +251,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
                 (__attribute__((address_space(3))) void*)(stage + BM * BKT + (r * ROWS_PER_IT + wave * RPI) * BKT), 16, 0, 0);
         }
     };
-
-    f32x16_t acc[MF][NF];
-#pragma unroll
-    for (int i = 0; i < MF; ++i)
-#pragma unroll
-        for (int j = 0; j < NF; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     // Fragment rows of a lane are (multiple of 32) + frow: the swizzle key is the same for all of them, so the
     // address is (row base + one per-k-step offset) + an immediate per fragment.
@@ -269,63 +270,89 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     for (int ks = 0; ks < KSTEPS; ++ks) pc[ks] = ((ks * 2 + fhalf) ^ key_f) << 4;
 
     const int k_tiles = K / BKT;
+    int tile = (int)blockIdx.x;
+    if (tile >= num_tiles) return;
+    set_tile(tile);
 #pragma unroll
     for (int s = 0; s < NSTAGE - 1; ++s)
         if (s < k_tiles) issue(s, lds + s * STAGE);
 
-    for (int kt = 0; kt < k_tiles; ++kt) {
-        // my share of tile kt has landed once at most the loads of the NSTAGE-2 younger tiles are outstanding
-        constexpr int kKeep = (NSTAGE - 2) * DMA_PER_TILE;
-        if (kt + NSTAGE - 2 < k_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (kKeep & 0xF) | ((kKeep >> 4) << 14));
-        else __builtin_amdgcn_s_waitcnt(0x0F70);
-        __builtin_amdgcn_s_barrier();     // everyone's share landed; everyone is done reading the stage reused below
-        if (kt + NSTAGE - 1 < k_tiles) issue(kt + NSTAGE - 1, lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE);
-        const char* stage = reinterpret_cast<const char*>(lds + (kt % NSTAGE) * STAGE);
-        Frag fa[KSTEPS][MF], fb[KSTEPS][NF];
+    Frag fa[KSTEPS][MF], fb[KSTEPS][NF];
+    while (true) {
+        f32x16_t acc[MF][NF];
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
+        for (int i = 0; i < MF; ++i)
 #pragma unroll
-            for (int i = 0; i < MF; ++i)
-                fa[ks][i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + i * 32 * BKT * (int)sizeof(T));
+            for (int j = 0; j < NF; ++j)
 #pragma unroll
-            for (int j = 0; j < NF; ++j) fb[ks][j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
-        }
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-            for (int i = 0; i < MF; ++i)
-#pragma unroll
-                for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks][i], fb[ks][j], acc[i][j]);
-    }
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // D fragment layout of v_mfma_f32_32x32x*: lane l, register v holds
-    //   row = 8*(v/4) + 4*(l/32) + (v%4)   (A / M index),   col = l%32   (B / N index)
-    if (EPI == kEpiSwiGLU) {
+        for (int kt = 0; kt < k_tiles; ++kt) {
+            // my share of tile kt has landed once at most the loads of the NSTAGE-2 younger tiles are outstanding
+            constexpr int kKeep = (NSTAGE - 2) * DMA_PER_TILE;
+            if (kt + NSTAGE - 2 < k_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (kKeep & 0xF) | ((kKeep >> 4) << 14));
+            else __builtin_amdgcn_s_waitcnt(0x0F70);
+            __builtin_amdgcn_s_barrier();     // everyone's share landed; everyone is done reading the stage reused below
+            if (kt + NSTAGE - 1 < k_tiles) issue(kt + NSTAGE - 1, lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE);
+            const char* stage = reinterpret_cast<const char*>(lds + (kt % NSTAGE) * STAGE);
 #pragma unroll
-        for (int i = 0; i < MF; ++i)
+            for (int ks = 0; ks < KSTEPS; ++ks) {
 #pragma unroll
-            for (int j = 0; j < NF / 2; ++j) {
-                const int col = n0 + wn * (WN / 2) + j * 32 + frow;
+                for (int i = 0; i < MF; ++i)
+                    fa[ks][i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + i * 32 * BKT * (int)sizeof(T));
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
-                    C[(int64_t)row * N + col] = Elem<T>::from_f32(silu_f32(acc[i][j][v]) * acc[i][j + NF / 2][v]);
-                }
+                for (int j = 0; j < NF; ++j) fb[ks][j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
             }
-    } else {
 #pragma unroll
-        for (int i = 0; i < MF; ++i)
+            for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
-            for (int j = 0; j < NF; ++j) {
-                const int col = n0 + wn * WN + j * 32 + frow;
+                for (int i = 0; i < MF; ++i)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int row = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
-                    float r = acc[i][j][v];
-                    if (R != nullptr) r += Elem<T>::to_f32(R[(int64_t)row * N + col]);
-                    C[(int64_t)row * N + col] = Elem<T>::from_f32(r);
+                    for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks][i], fb[ks][j], acc[i][j]);
+        }
+
+        // start the next tile's first stages before this tile's epilogue, so that its global-load latency is covered
+        const int out_m0 = m0, out_n0 = n0;
+        const int next = tile + (int)gridDim.x;
+        if (next < num_tiles) {
+            set_tile(next);
+            __builtin_amdgcn_s_barrier();     // every wave has issued its reads of the last stage
+#pragma unroll
+            for (int s = 0; s < NSTAGE - 1; ++s)
+                if (s < k_tiles) issue(s, lds + s * STAGE);
+        }
+
+        // D fragment layout of v_mfma_f32_32x32x*: lane l, register v holds
+        //   row = 8*(v/4) + 4*(l/32) + (v%4)   (A / M index),   col = l%32   (B / N index)
+        if (EPI == kEpiSwiGLU) {
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+                for (int j = 0; j < NF / 2; ++j) {
+                    const int col = out_n0 + wn * (WN / 2) + j * 32 + frow;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = out_m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
+                        C[(int64_t)row * N + col] = Elem<T>::from_f32(silu_f32(acc[i][j][v]) * acc[i][j + NF / 2][v]);
+                    }
                 }
-            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+                for (int j = 0; j < NF; ++j) {
+                    const int col = out_n0 + wn * WN + j * 32 + frow;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = out_m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
+                        float r = acc[i][j][v];
+                        if (R != nullptr) r += Elem<T>::to_f32(R[(int64_t)row * N + col]);
+                        C[(int64_t)row * N + col] = Elem<T>::from_f32(r);
+                    }
+                }
+        }
+        if (next >= num_tiles) break;
+        tile = next;
     }
 }
 
@@ -396,9 +423,14 @@ template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NST
 void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
     const int tiles_m = M / BM, tiles_n = N / BN_OUT;
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI>),
-                       dim3((unsigned)(tiles_m * tiles_n)), dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N,
-                       K, tiles_m, tiles_n);
+    // persistent workgroups: as many as are resident at once (LDS-limited), a multiple of 8 so that the XCD patches hold
+    constexpr int kStageBytes = (BM + BN) * BKT * (int)sizeof(T) * NSTAGE;
+    constexpr int kPerCu = (160 * 1024 / kStageBytes) < 1 ? 1 : ((160 * 1024 / kStageBytes) > 2 ? 2 : (160 * 1024 / kStageBytes));
+    const int total = tiles_m * tiles_n;
+    const int resident = 256 * kPerCu;
+    const int grid = total < resident ? total : resident;
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI>), dim3((unsigned)grid),
+                       dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
 }
 
 // Tile choice: 256-wide tiles (8 waves) halve the LDS traffic per MFMA but need >= 256 of them to occupy the chip;

@@ -142,7 +142,8 @@ __device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_group
 template <typename T, typename TG, int RK, bool FROM_LOGITS>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
     const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
-    int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob) {
+    int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets,
+    uint32_t row_bytes) {
     constexpr int KP = RK * kWave;
     __shared__ uint16_t cand[kMaxCand];
     __shared__ float half_score[kRouterWaves][2][KP];
@@ -223,6 +224,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
                     const int64_t o = token * top_k + p;
                     scores[o] = Elem<T>::from_f32(key_score(best[r]));
                     indices[o] = (int64_t)key_index(best[r]);
+                    if (row_offsets != nullptr) row_offsets[o] = key_index(best[r]) * row_bytes;
                     if (gates != nullptr) gates[o] = Elem<TG>::from_f32(norm_topk_prob ? e[r] / total : e[r]);
                 }
             }
@@ -239,7 +241,7 @@ int count_candidates(int top_k) {
 
 template <typename T, typename TG, bool FROM_LOGITS>
 int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64_t* indices, void* gates,
-                  int norm, hipStream_t stream) {
+                  int norm, uint32_t* row_offsets, uint32_t row_bytes, hipStream_t stream) {
     const int num_cand = count_candidates(K);
     const int64_t blocks_needed = (T_ + kRouterWaves - 1) / kRouterWaves;
     const int64_t max_blocks = 256 * 8;   // a few resident blocks per CU; the kernel loops over tokens
@@ -247,7 +249,7 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
     const dim3 block(kRouterWaves * kWave);
 #define FMOE_LAUNCH_ROUTER(R)                                                                                      \
     hipLaunchKernelGGL((router_topk_kernel<T, TG, R, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, T_, nk, K, \
-                       num_cand, (T*)scores, indices, (TG*)gates, norm)
+                       num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes)
     if (K <= 64) FMOE_LAUNCH_ROUTER(1);
     else if (K <= 128) FMOE_LAUNCH_ROUTER(2);
     else FMOE_LAUNCH_ROUTER(4);
@@ -259,11 +261,12 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
 }  // namespace
 
 int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
-                              int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, hipStream_t stream) {
+                              int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, uint32_t* row_offsets,
+                              uint32_t row_bytes, hipStream_t stream) {
     switch (gate_dtype) {
-        case FMOE_F32: return launch_router<float, float, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, stream);
-        case FMOE_BF16: return launch_router<float, bf16_t, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, stream);
-        default: return launch_router<float, f16_t, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, stream);
+        case FMOE_F32: return launch_router<float, float, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, row_offsets, row_bytes, stream);
+        case FMOE_BF16: return launch_router<float, bf16_t, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, row_offsets, row_bytes, stream);
+        default: return launch_router<float, f16_t, true>(logits, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, row_offsets, row_bytes, stream);
     }
 }
 
@@ -284,8 +287,8 @@ extern "C" int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int n
     FMOE_REQUIRE(log_probs && scores && indices, FMOE_ERR_NULL_POINTER, "fmoe_router_topk: null tensor pointer");
     hipStream_t s = (hipStream_t)stream;
     switch (dtype) {
-        case FMOE_F32: return launch_router<float, float, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
-        case FMOE_BF16: return launch_router<bf16_t, bf16_t, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
-        default: return launch_router<f16_t, f16_t, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, s);
+        case FMOE_F32: return launch_router<float, float, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, nullptr, 0u, s);
+        case FMOE_BF16: return launch_router<bf16_t, bf16_t, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, nullptr, 0u, s);
+        default: return launch_router<f16_t, f16_t, false>(log_probs, num_tokens, num_keys, top_k, scores, indices, gates, norm_topk_prob, nullptr, 0u, s);
     }
 }

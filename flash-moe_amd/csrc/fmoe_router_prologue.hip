@@ -400,8 +400,20 @@ extern "C" int fmoe_router_forward(const void* x, const void* gate_w, void* runn
                                    float eps, int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype,
                                    int norm_topk_prob, void* router_logits, float* logits_fp32, float* scores,
                                    int64_t* indices, void* gates, void* workspace, size_t workspace_bytes, void* stream) {
+    fmoe::clear_error();
+    return fmoe::router_forward_impl(x, gate_w, running_mean, running_var, num_batches_tracked, stats_dtype, training,
+                                     momentum, eps, num_tokens, hidden, num_keys, top_k, dtype, norm_topk_prob,
+                                     router_logits, logits_fp32, scores, indices, gates, nullptr, 0u, workspace,
+                                     workspace_bytes, (hipStream_t)stream);
+}
+
+int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_mean, void* running_var,
+                              int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
+                              int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
+                              void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
+                              uint32_t* row_offsets, uint32_t row_bytes, void* workspace, size_t workspace_bytes,
+                              hipStream_t s) {
     using namespace fmoe;
-    clear_error();
     FMOE_REQUIRE(dtype_ok(dtype) && dtype_ok(stats_dtype), FMOE_ERR_BAD_DTYPE,
                  "fmoe_router_forward: unknown dtype %d / statistics dtype %d", dtype, stats_dtype);
     FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_keys > 0, FMOE_ERR_BAD_SHAPE,
@@ -427,7 +439,6 @@ extern "C" int fmoe_router_forward(const void* x, const void* gate_w, void* runn
     const ProloguePlan p = plan_prologue(num_tokens, hidden, num_keys);
     FMOE_REQUIRE(workspace_bytes >= p.bytes && aligned16(workspace), FMOE_ERR_WORKSPACE,
                  "fmoe_router_forward: workspace of %zu bytes needed, %zu given", p.bytes, workspace_bytes);
-    hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
     float* partial = (float*)(ws + p.off_partial);
     float* mean_rstd = (float*)(ws + p.off_mean_rstd);
@@ -466,5 +477,6 @@ extern "C" int fmoe_router_forward(const void* x, const void* gate_w, void* runn
     }
     FMOE_CHECK_LAUNCH("fmoe_router_forward(gate)");
     if (top_k == 0) return FMOE_OK;
-    return launch_router_from_logits(logits32, num_tokens, num_keys, top_k, scores, indices, gates, dtype, norm_topk_prob, s);
+    return launch_router_from_logits(logits32, num_tokens, num_keys, top_k, scores, indices, gates, dtype, norm_topk_prob,
+                                     row_offsets, row_bytes, s);
 }

@@ -38,6 +38,9 @@ SIGNATURES = {
     "fmoe_expert_forward_algo": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _int, _vp]),
     "fmoe_mlp_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
     "fmoe_mlp_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp, _sz, _vp]),
+    "fmoe_block_workspace_bytes": (_sz, [_i64, _int, _int, _int, _i64, _int, _int]),
+    "fmoe_block_forward": (_int, [_vp] * 10 + [_int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int, _i64, _int, _int,
+                                  _int, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_mlp_gate_up": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
     "fmoe_mlp_down": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp]),
 }

@@ -5,11 +5,12 @@ six arguments (flash_moe/modules/flash_moe.py:12-27), ``FlashMoE`` owns paramete
 the same ``state_dict`` names (:43-53) and ``forward`` returns the same ``(hidden_states, router_logits)``
 pair (:55-105).
 
-Stages of ``forward``, all HIP:
+``forward`` is one call of ``fmoe_block_forward``, whose stages are those of the per-op entry points:
   batch-norm, router gate, log-softmax, product-key top-k, gates    ``fmoe_router_forward``
   routed experts                                                    ``fmoe_expert_forward``
   shared SwiGLU MLP + add                                           ``fmoe_mlp_forward`` (the add is the second
                                                                     GEMM's epilogue)
+``forward_staged`` runs the same three stages as three calls.
 
 Routing is evaluated in fp32 whatever the module dtype: the normalised activations are rounded to the
 module dtype exactly as the reference does, but their product with the router gate, the log-softmax
@@ -26,6 +27,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from flash_moe.ops.hip.flash_block import block_forward
 from flash_moe.ops.hip.flash_expert import expert_forward
 from flash_moe.ops.hip.flash_mlp import mlp_forward
 from flash_moe.ops.hip.flash_router import router_forward
@@ -85,7 +87,18 @@ class FlashMoE(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, **kwargs):
         bsz, seq_len, _ = hidden_states.shape
-        tokens = hidden_states.view(-1, self.hidden_size)
+        tokens = hidden_states.reshape(-1, self.hidden_size)
+        out, logits = block_forward(
+            tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, self.router_gate.weight,
+            self.router_norm, self.down_embed.weight, self.up_embed.weight, self.num_keys, self.top_k, self.norm_topk_prob,
+        )
+        router_logits = logits.view(tokens.shape[0], 2, self.num_keys).transpose(0, 1)
+        return out.view(bsz, seq_len, -1), router_logits
+
+    def forward_staged(self, hidden_states: torch.Tensor):
+        """``forward`` as three library calls (router, experts, MLP) instead of one; same results."""
+        bsz, seq_len, _ = hidden_states.shape
+        tokens = hidden_states.reshape(-1, self.hidden_size)
         router_logits, _, indices, gates = self.route(tokens)
         experts_states = expert_forward(tokens, self.down_embed.weight, self.up_embed.weight, indices, gates)
         out = mlp_forward(

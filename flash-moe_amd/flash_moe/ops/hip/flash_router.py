@@ -54,15 +54,8 @@ def router_topk_gates(
     return scores, indices, gates
 
 
-def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.nn.BatchNorm1d, num_expert_keys: int,
-                   num_experts_per_tok: int, norm_topk_prob: bool = False, return_logits32: bool = False):
-    """The block's whole routing stage in one call of ``fmoe_router_forward``: batch-norm (training or evaluation
-    mode, taken from ``norm.training``; its running statistics are updated in place), the router gate, the per-half
-    log-softmax, the product-key top-k and the gates (flash_moe/modules/flash_moe.py:62-85).
-
-    Returns ``(router_logits [T, 2*nk] in tokens.dtype, scores [T,K] fp32, indices [T,K] int64, gates [T,K] in
-    tokens.dtype)``, plus the fp32 logits the routing was computed from when ``return_logits32`` is set.
-    """
+def check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok):
+    """Argument checks of the fused routing stage; returns ``(device, training)``."""
     if tokens.dim() != 2 or gate_weight.shape != (2 * num_expert_keys, tokens.shape[1]):
         raise ValueError("expected tokens [T, H] and a router gate weight [2*num_expert_keys, H]")
     assert 0 <= num_experts_per_tok <= num_expert_keys, (
@@ -73,10 +66,25 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
     if norm.affine or norm.momentum is None or not norm.track_running_stats:
         raise ValueError("the fused router expects BatchNorm1d(affine=False, momentum=<float>, track_running_stats=True)")
     training = bool(norm.training)
-    T, H = tokens.shape
-    if training and T == 1:
+    if training and tokens.shape[0] == 1:
         raise ValueError(f"Expected more than 1 value per channel when training, got input size {tuple(tokens.shape)}")
-    dev = _C.require_gpu(tokens, gate_weight, norm.running_mean, norm.running_var)
+    rm, rv = norm.running_mean, norm.running_var
+    if not (rm.is_contiguous() and rv.is_contiguous() and rm.dtype == rv.dtype):
+        raise ValueError("running statistics must be contiguous and of one dtype")
+    return _C.require_gpu(tokens, gate_weight, rm, rv), training
+
+
+def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.nn.BatchNorm1d, num_expert_keys: int,
+                   num_experts_per_tok: int, norm_topk_prob: bool = False, return_logits32: bool = False):
+    """The block's whole routing stage in one call of ``fmoe_router_forward``: batch-norm (training or evaluation
+    mode, taken from ``norm.training``; its running statistics are updated in place), the router gate, the per-half
+    log-softmax, the product-key top-k and the gates (flash_moe/modules/flash_moe.py:62-85).
+
+    Returns ``(router_logits [T, 2*nk] in tokens.dtype, scores [T,K] fp32, indices [T,K] int64, gates [T,K] in
+    tokens.dtype)``, plus the fp32 logits the routing was computed from when ``return_logits32`` is set.
+    """
+    dev, training = check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok)
+    T, H = tokens.shape
     x, w = tokens.contiguous(), gate_weight.contiguous()
     K = num_experts_per_tok
     logits = torch.empty((T, 2 * num_expert_keys), device=dev, dtype=x.dtype)
@@ -88,8 +96,6 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
     ws_bytes = L.fmoe_router_workspace_bytes(T, H, num_expert_keys)
     ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
     rm, rv, nbt = norm.running_mean, norm.running_var, norm.num_batches_tracked
-    if not (rm.is_contiguous() and rv.is_contiguous() and rm.dtype == rv.dtype):
-        raise ValueError("running statistics must be contiguous and of one dtype")
     with torch.cuda.device(dev):
         status = L.fmoe_router_forward(
             _C.ptr(x), _C.ptr(w), _C.ptr(rm), _C.ptr(rv), _C.ptr(nbt), _C.dtype_code(rm.dtype), int(training),

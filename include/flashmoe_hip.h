@@ -157,6 +157,28 @@ int fmoe_mlp_gate_up(const void* x, const void* gate_w, const void* up_w, int64_
 int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int hidden, int intermediate, int dtype,
                   const void* residual, void* out, void* stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * The whole block: FlashMoE.forward (flash_moe/modules/flash_moe.py:55-105) in one call, on the flattened tokens.
+ *   out = mlp(x) + experts(x, route(x)),   router_logits = router_gate(router_norm(x))
+ * Same stages and numerics as fmoe_router_forward -> fmoe_expert_forward -> fmoe_mlp_forward(residual = experts);
+ * intermediates live in `workspace` (fmoe_block_workspace_bytes(), 256-byte aligned).
+ *
+ *   x [T,H]; gate_proj_w, up_proj_w [I,H]; down_proj_w [H,I]; router_gate_w [2*nk,H]; down_embed, up_embed [E,H]: dtype
+ *   running_mean / running_var / num_batches_tracked, stats_dtype, training, momentum, eps: as in fmoe_router_forward
+ *   out [T,H] dtype; router_logits [T,2*nk] dtype
+ *   indices_out [T,K] int64 and gates_out [T,K] dtype: optional (NULL keeps them in the workspace)
+ * Requires nk*nk <= E and 0 <= top_k <= nk.
+ */
+size_t fmoe_block_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int num_keys, int64_t num_experts,
+                                  int top_k, int dtype);
+
+int fmoe_block_forward(const void* x, const void* gate_proj_w, const void* up_proj_w, const void* down_proj_w,
+                       const void* router_gate_w, const void* down_embed, const void* up_embed, void* running_mean,
+                       void* running_var, int64_t* num_batches_tracked, int stats_dtype, int training, float momentum,
+                       float eps, int64_t num_tokens, int hidden, int intermediate, int64_t num_experts, int num_keys,
+                       int top_k, int dtype, int norm_topk_prob, void* out, void* router_logits, int64_t* indices_out,
+                       void* gates_out, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

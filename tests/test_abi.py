@@ -113,6 +113,33 @@ def test_mlp_argument_checks():
     assert f(None, None, None, None, 0, 64, 128, _C.BF16, None, None, None, 0, None) == 0
 
 
+def test_block_argument_checks():
+    lib = _C.lib()
+    keep, a = _buf()
+    f = lib.fmoe_block_forward
+    T, H, I, E, nk, K = 8, 64, 128, 1024, 32, 4
+    need = lib.fmoe_block_workspace_bytes(T, H, I, nk, E, K, _C.BF16)
+    parts = (lib.fmoe_router_workspace_bytes(T, H, nk) + lib.fmoe_expert_workspace_bytes(T, H, E, K, _C.BF16)
+             + lib.fmoe_mlp_workspace_bytes(T, H, I, _C.BF16))
+    assert need >= parts + T * 2 * nk * 4 + T * K * (4 + 8 + 2) + T * H * 2 and need % 256 == 0
+    assert lib.fmoe_block_workspace_bytes(T, H, I, nk, E, K, 9) == 0
+
+    def call(T=T, H=H, I=I, E=E, nk=nk, K=K, dtype=_C.BF16, x=a, ws=a, ws_bytes=need):
+        return f(x, a, a, a, a, a, a, a, a, a, _C.F32, 1, 0.1, 1e-5, T, H, I, E, nk, K, dtype, 0, a, a, None, None,
+                 ws, ws_bytes, None)
+
+    assert call(dtype=6) == -4
+    assert call(I=0) == -2
+    assert call(nk=33) == -2                      # nk*nk > E
+    assert call(K=33) == -3 and b"[0, 32]" in lib.fmoe_last_error()
+    assert call(x=None) == -1
+    assert call(H=60) == -6
+    assert call(I=100) == -6
+    assert call(ws_bytes=need - 1) == -7
+    assert call(ws=None) == -7
+    assert call(T=0, x=None, ws=None, ws_bytes=0) == 0
+
+
 def test_python_wrappers_refuse_cpu_tensors():
     from flash_moe.ops import flash_expert_func, flash_mlp_func, flash_router_func
 

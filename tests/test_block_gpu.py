@@ -125,3 +125,42 @@ def test_block_c5_shape_fewer_tokens():
     m, w = build(2048, 8192, 262144, 128, True, dtype)
     x = torch.randn(1, 256, 2048, generator=torch.Generator().manual_seed(0)).to(dtype)
     stagewise_check(m, w, x, 128, True, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,I,E,K", [(1024, 256, 512, 4096, 32),     # column-slice expert schedule
+                                       (96, 128, 256, 1024, 8),        # row-gather expert schedule
+                                       (33, 64, 192, 400, 5)])         # ragged: E not a square, odd T and K
+@pytest.mark.parametrize("training", [True, False])
+def test_single_call_block_equals_the_three_stage_calls(dtype, T, H, I, E, K, training):
+    """fmoe_block_forward runs the same kernels as router -> expert -> mlp called one by one: bit-identical."""
+    from flash_moe.ops.hip.flash_block import block_forward
+
+    m, _ = build(H, I, E, K, True, dtype, seed=3)
+    m.train(training)
+    x = torch.randn(1, T, H, generator=torch.Generator().manual_seed(5)).to(dtype).cuda()
+    y1, l1 = m(x)
+    stats1 = (m.router_norm.running_mean.clone(), m.router_norm.running_var.clone(), int(m.router_norm.num_batches_tracked))
+    m.router_norm.reset_running_stats()
+    y2, l2 = m.forward_staged(x)
+    assert torch.equal(y1, y2) and torch.equal(l1, l2)
+    assert torch.equal(stats1[0], m.router_norm.running_mean) and torch.equal(stats1[1], m.router_norm.running_var)
+    assert stats1[2] == int(m.router_norm.num_batches_tracked) == (1 if training else 0)
+    m.router_norm.reset_running_stats()
+    _, _, idx_ref, gates_ref = m.route(x.view(T, H))
+    m.router_norm.reset_running_stats()
+    y3, _, idx, gates = block_forward(x.view(T, H), m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight,
+                                      m.router_gate.weight, m.router_norm, m.down_embed.weight, m.up_embed.weight,
+                                      m.num_keys, K, True, return_routing=True)
+    assert torch.equal(idx, idx_ref) and torch.equal(gates, gates_ref) and torch.equal(y3.view_as(y1), y1)
+
+
+def test_single_call_block_without_routed_experts():
+    """num_experts_per_tok = 0: the block is the shared MLP alone."""
+    from flash_moe.ops.hip.flash_mlp import mlp_forward
+
+    m, _ = build(128, 256, 1024, 0, False, torch.bfloat16, seed=1)
+    x = torch.randn(2, 32, 128, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
+    y, logits = m(x)
+    ref = mlp_forward(x.view(-1, 128), m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight)
+    assert torch.equal(y.view(-1, 128), ref) and logits.shape == (2, 64, 32)
