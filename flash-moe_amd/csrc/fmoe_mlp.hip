@@ -29,6 +29,7 @@ constexpr int BK = kTileK;        // k extent of a register-staged LDS tile (ele
 constexpr int kChunksPerRow = kTileChunks;
 
 enum Epilogue { kEpiSwiGLU = 0, kEpiPlain = 1 };
+template <bool B> struct Flag { static constexpr bool value = B; };
 
 template <typename T, int BM, int BN, int EPI>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
 // ------------------------------------------------------------------------------------------------------------
 // LDS-DMA pipelined kernel.  WAVES_M x WAVES_N waves, each (BM/WAVES_M) x (BN/WAVES_N); BKT = k extent of a stage.
 // ------------------------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
     const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n) {
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     // key does not depend on the round and one element offset per lane serves every load.
     const int lrow = lane / CPR, lp = lane % CPR;
     const int key_dma = ((wave * RPI + lrow) >> ROW_SHIFT) & (CPR - 1);
-    const int lane_off = lrow * K + ((lp ^ key_dma) << 3);
+    const uint32_t lane_off = (uint32_t)(lrow * K + ((lp ^ key_dma) << 3)) * (uint32_t)sizeof(T);   // bytes
     const T *a_src, *b_src0, *b_src1 = nullptr;
     int m0, n0;
     // The workgroup is persistent: it takes tiles t, t + gridDim.x, ...  Each XCD (workgroup id mod 8) gets a contiguous
@@ -230,16 +231,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
         m0 = (first_m + (t % width) % gsz) * BM;
         n0 = ((t % width) / gsz) * BN_OUT;
-        a_src = A + (int64_t)(m0 + wave * RPI) * K + lane_off;
-        b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K + lane_off;
-        if (EPI == kEpiSwiGLU) b_src1 = B1 + (int64_t)(n0 + wave * RPI) * K + lane_off;
+        a_src = A + (int64_t)(m0 + wave * RPI) * K;      // wave-uniform; the lane's part is the 32-bit lane_off
+        b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K;
+        if (EPI == kEpiSwiGLU) b_src1 = B1 + (int64_t)(n0 + wave * RPI) * K;
     };
     auto issue = [&](int kt, T* stage) {
         const int k0 = kt * BKT;
 #pragma unroll
         for (int r = 0; r < A_ROUNDS; ++r)
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(a_src + (int64_t)r * ROWS_PER_IT * K + k0),
+                (const __attribute__((address_space(1))) void*)((const char*)(a_src + (int64_t)r * ROWS_PER_IT * K + k0) + lane_off),
                 (__attribute__((address_space(3))) void*)(stage + (r * ROWS_PER_IT + wave * RPI) * BKT), 16, 0, 0);
 #pragma unroll
         for (int r = 0; r < B_ROUNDS; ++r) {
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
             if (EPI == kEpiSwiGLU && r >= B_ROUNDS / 2) src = b_src1 + (int64_t)(r - B_ROUNDS / 2) * ROWS_PER_IT * K + k0;
             else src = b_src0 + (int64_t)r * ROWS_PER_IT * K + k0;
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)src,
+                (const __attribute__((address_space(1))) void*)((const char*)src + lane_off),
                 (__attribute__((address_space(3))) void*)(stage + BM * BKT + (r * ROWS_PER_IT + wave * RPI) * BKT), 16, 0, 0);
         }
     };
@@ -277,7 +278,30 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     for (int s = 0; s < NSTAGE - 1; ++s)
         if (s < k_tiles) issue(s, lds + s * STAGE);
 
-    Frag fa[KSTEPS][MF], fb[KSTEPS][NF];
+    // Fragments of k-step ks+PF are read from LDS while the MFMAs of k-step ks run (PF+1 register buffers); the
+    // read-ahead crosses k-tile boundaries, so the barrier that publishes the next stage sits PF k-steps before the
+    // end of a k-tile and the matrix pipe always has work queued while a wave waits.
+    constexpr int RING = PF + 1;
+    static_assert(KSTEPS % RING == 0 && PF >= 1 && PF < KSTEPS + 1, "fragment buffers rotate with period RING");
+    Frag fa[RING][MF], fb[RING][NF];
+    auto read_frags = [&](const char* stage, int ks, Frag (&a)[MF], Frag (&b)[NF]) {
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+            a[i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + i * 32 * BKT * (int)sizeof(T));
+#pragma unroll
+        for (int j = 0; j < NF; ++j) b[j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
+    };
+    // Entering k-tile kt (kt = 0: from the tile prologue): my share of its stage has landed once at most the loads of
+    // the NSTAGE-2 younger k-tiles are outstanding; my reads of the stage that is overwritten next are complete (all
+    // reads of k-tile kt-1 have been issued by then); after the barrier both hold for every wave, so the load of k-tile
+    // kt+NSTAGE-1 can go into the stage kt-1 used.
+    auto enter_k_tile = [&](int kt) {
+        constexpr int kKeep = (NSTAGE - 2) * DMA_PER_TILE;
+        if (kt + NSTAGE - 2 < k_tiles) __builtin_amdgcn_s_waitcnt(0x0070 | (kKeep & 0xF) | ((kKeep >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0070);
+        __builtin_amdgcn_s_barrier();
+        if (kt + NSTAGE - 1 < k_tiles) issue(kt + NSTAGE - 1, lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE);
+    };
     while (true) {
         f32x16_t acc[MF][NF];
 #pragma unroll
@@ -287,36 +311,52 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-        for (int kt = 0; kt < k_tiles; ++kt) {
-            // my share of tile kt has landed once at most the loads of the NSTAGE-2 younger tiles are outstanding
-            constexpr int kKeep = (NSTAGE - 2) * DMA_PER_TILE;
-            if (kt + NSTAGE - 2 < k_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (kKeep & 0xF) | ((kKeep >> 4) << 14));
-            else __builtin_amdgcn_s_waitcnt(0x0F70);
-            __builtin_amdgcn_s_barrier();     // everyone's share landed; everyone is done reading the stage reused below
-            if (kt + NSTAGE - 1 < k_tiles) issue(kt + NSTAGE - 1, lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE);
+        enter_k_tile(0);
+#pragma unroll
+        for (int s = 0; s < PF; ++s) read_frags(reinterpret_cast<const char*>(lds), s, fa[s], fb[s]);
+        // the last k-tile has no successor to read ahead into: it is a separate copy of the body, so that no branch
+        // merges a path with reads in flight into the MFMA sequence
+        auto k_tile_body = [&](int kt, auto last_tag) {
+            constexpr bool kLast = decltype(last_tag)::value;
             const char* stage = reinterpret_cast<const char*>(lds + (kt % NSTAGE) * STAGE);
+            const char* next_stage = reinterpret_cast<const char*>(lds + ((kt + 1) % NSTAGE) * STAGE);
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
+                constexpr int kReads = MF + NF, kMfmas = MF * NF;
+                const int nxt = ks + PF;
+                const bool reads = nxt < KSTEPS || !kLast;
+                __builtin_amdgcn_sched_barrier(0);
+                if (nxt < KSTEPS) {
+                    read_frags(stage, nxt, fa[nxt % RING], fb[nxt % RING]);
+                } else if (!kLast) {
+                    if (nxt == KSTEPS) {
+                        enter_k_tile(kt + 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    read_frags(next_stage, nxt - KSTEPS, fa[nxt % RING], fb[nxt % RING]);
+                }
 #pragma unroll
                 for (int i = 0; i < MF; ++i)
-                    fa[ks][i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + i * 32 * BKT * (int)sizeof(T));
 #pragma unroll
-                for (int j = 0; j < NF; ++j) fb[ks][j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
+                    for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks % RING][i], fb[ks % RING][j], acc[i][j]);
+                static_assert(kReads <= kMfmas, "one LDS read after each of the first MFMAs");
+#pragma unroll
+                for (int q = 0; q < kMfmas; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (reads && q < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
             }
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-                for (int i = 0; i < MF; ++i)
-#pragma unroll
-                    for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks][i], fb[ks][j], acc[i][j]);
-        }
+        };
+        for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile_body(kt, Flag<false>{});
+        k_tile_body(k_tiles - 1, Flag<true>{});
+        __builtin_amdgcn_sched_barrier(0);
 
         // start the next tile's first stages before this tile's epilogue, so that its global-load latency is covered
         const int out_m0 = m0, out_n0 = n0;
         const int next = tile + (int)gridDim.x;
         if (next < num_tiles) {
             set_tile(next);
-            __builtin_amdgcn_s_barrier();     // every wave has issued its reads of the last stage
+            __builtin_amdgcn_s_barrier();     // every wave has consumed its reads of the last stage
 #pragma unroll
             for (int s = 0; s < NSTAGE - 1; ++s)
                 if (s < k_tiles) issue(s, lds + s * STAGE);
@@ -324,31 +364,43 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 
         // D fragment layout of v_mfma_f32_32x32x*: lane l, register v holds
         //   row = 8*(v/4) + 4*(l/32) + (v%4)   (A / M index),   col = l%32   (B / N index)
+        // Buffer addressing: a wave-uniform descriptor of the rows from the wave's first one on, a scalar byte offset
+        // per (fragment, register) and one 32-bit byte offset per lane - no vector address arithmetic per element.
+        const int lane_bytes = ((4 * fhalf) * N + frow) * (int)sizeof(T);
+        const int64_t wave_off = (int64_t)(out_m0 + wm * WM) * N + out_n0 + wn * ((EPI == kEpiSwiGLU) ? WN / 2 : WN);
+        const int64_t span = ((int64_t)M * N - wave_off) * (int64_t)sizeof(T);
+        const int span32 = (int)(span < 0x7FFFFFFFll ? span : 0x7FFFFFFFll);
+        auto c_rsrc = __builtin_amdgcn_make_buffer_rsrc(C + wave_off, 0, span32, 0x00020000);
+        auto store_elem = [&](int uni_bytes, float value) {
+            const T t = Elem<T>::from_f32(value);
+            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, t), c_rsrc, lane_bytes, uni_bytes, 0);
+        };
         if (EPI == kEpiSwiGLU) {
 #pragma unroll
             for (int i = 0; i < MF; ++i)
 #pragma unroll
-                for (int j = 0; j < NF / 2; ++j) {
-                    const int col = out_n0 + wn * (WN / 2) + j * 32 + frow;
+                for (int j = 0; j < NF / 2; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int row = out_m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
-                        C[(int64_t)row * N + col] = Elem<T>::from_f32(silu_f32(acc[i][j][v]) * acc[i][j + NF / 2][v]);
-                    }
-                }
+                    for (int v = 0; v < 16; ++v)
+                        store_elem(((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T),
+                                   silu_fast_f32(acc[i][j][v]) * acc[i][j + NF / 2][v]);
         } else {
+            auto r_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(R != nullptr ? R + wave_off : C), 0,
+                                                            R != nullptr ? span32 : 0, 0x00020000);   // no residual: reads give 0
 #pragma unroll
             for (int i = 0; i < MF; ++i)
 #pragma unroll
                 for (int j = 0; j < NF; ++j) {
-                    const int col = out_n0 + wn * WN + j * 32 + frow;
+                    float res[16];
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        const int row = out_m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * fhalf + (v % 4);
-                        float r = acc[i][j][v];
-                        if (R != nullptr) r += Elem<T>::to_f32(R[(int64_t)row * N + col]);
-                        C[(int64_t)row * N + col] = Elem<T>::from_f32(r);
+                        const int uni = ((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T);
+                        const short raw = __builtin_amdgcn_raw_buffer_load_b16(r_rsrc, lane_bytes, uni, 0);
+                        res[v] = Elem<T>::to_f32(__builtin_bit_cast(T, raw));
                     }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        store_elem(((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T), acc[i][j][v] + res[v]);
                 }
         }
         if (next >= num_tiles) break;
@@ -419,7 +471,7 @@ void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, 
                        stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
 void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
     const int tiles_m = M / BM, tiles_n = N / BN_OUT;
@@ -429,20 +481,28 @@ void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int
     const int total = tiles_m * tiles_n;
     const int resident = 256 * kPerCu;
     const int grid = total < resident ? total : resident;
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI>), dim3((unsigned)grid),
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI, PF>), dim3((unsigned)grid),
                        dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
 }
 
-// Tile choice: 256-wide tiles (8 waves) halve the LDS traffic per MFMA but need >= 256 of them to occupy the chip;
-// otherwise 128x128 tiles (4 waves, two workgroups per CU).
+// Tile choice: 256-wide tiles (8 waves, two per SIMD) halve the L2 -> LDS traffic per MFMA but need >= 256 of them to
+// occupy the chip; otherwise 128x128 tiles of 4 waves, which read a whole k-tile of fragments ahead (PF = 3): one
+// workgroup per CU with four stages in flight when every tile gets a CU of its own, two per CU with two stages else.
+template <typename T, int EPI>
+void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, int64_t tiles,
+                        hipStream_t stream) {
+    if (tiles <= 256) launch_gemm_dma<T, 128, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+    else launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+}
+
 template <typename T>
 int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, hipStream_t stream) {
     const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu;
     const bool k_ok = H % 64 == 0;
     if (k_ok && M % 256 == 0 && I % 128 == 0 && (int64_t)(M / 256) * (I / 128) >= 256)
-        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, nullptr, M, I, H, stream);
     else if (k_ok && M % 128 == 0 && I % 64 == 0)
-        launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
+        launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, (int64_t)(M / 128) * (I / 64), stream);
     else
         launch_gemm<T, 128, 128, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up)");
@@ -454,9 +514,9 @@ int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* r
     const T *A = (const T*)h, *W = (const T*)wd, *R = (const T*)residual;
     const bool k_ok = I % 64 == 0;
     if (k_ok && M % 256 == 0 && H % 256 == 0 && (int64_t)(M / 256) * (H / 256) >= 256)
-        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiPlain, 1>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     else if (k_ok && M % 128 == 0 && H % 128 == 0)
-        launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
+        launch_small_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, (int64_t)(M / 128) * (H / 128), stream);
     else
         launch_gemm<T, 128, 128, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(down)");
