@@ -36,6 +36,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 
 C4 = dict(batch=1, seq=4096, hidden=1024, inter=4096, experts=16384, top_k=64, norm=False)
 C3 = dict(tokens=16384, hidden=1024, experts=16384, top_k=64)
+C2 = dict(tokens=8192, hidden=1024, keys=128, top_k=64)
+C5 = dict(batch=8, seq=4096, hidden=2048, inter=8192, experts=262144, top_k=128, norm=True)
 
 
 def log(*a):
@@ -215,6 +217,73 @@ def bench_expert_c3(dtype, iters):
                 tokens_per_s=round(T / (ms * 1e-3)), traffic=measured_traffic("expert", "c3"))
 
 
+def bench_router_c2(dtype, iters):
+    """The routing stage alone on its own shape: the fused call (batch norm, gate, log-softmax, top-k, gates) and the
+    top-k op on ready-made fp32 log-probabilities."""
+    import torch
+
+    from flash_moe import _C
+
+    T, H, nk, K = C2["tokens"], C2["hidden"], C2["keys"], C2["top_k"]
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(T, H, generator=g).to(dtype).cuda()
+    w = (torch.randn(2 * nk, H, generator=g) * 0.02).to(dtype).cuda()
+    lp = torch.log_softmax(torch.randn(2, T, nk, generator=g), -1).cuda()
+    L = _C.lib()
+    code = _C.dtype_code(dtype)
+    logits = torch.empty(T, 2 * nk, device="cuda", dtype=dtype)
+    logits32 = torch.empty(T, 2 * nk, device="cuda", dtype=torch.float32)
+    scores = torch.empty(T, K, device="cuda", dtype=torch.float32)
+    indices = torch.empty(T, K, device="cuda", dtype=torch.int64)
+    gates = torch.empty(T, K, device="cuda", dtype=dtype)
+    ws_bytes = L.fmoe_router_workspace_bytes(T, H, nk)
+    ws = torch.empty(max(ws_bytes, 1), device="cuda", dtype=torch.uint8)
+    stream = lambda: _C.current_stream(x.device)
+
+    def fused():
+        rc = L.fmoe_router_forward(x.data_ptr(), w.data_ptr(), None, None, None, code, 1, 0.1, 1e-5, T, H, nk, K, code, 0,
+                                   logits.data_ptr(), logits32.data_ptr(), scores.data_ptr(), indices.data_ptr(),
+                                   gates.data_ptr(), ws.data_ptr(), ws_bytes, stream())
+        if rc:
+            raise RuntimeError(L.fmoe_last_error().decode())
+
+    def topk():
+        rc = L.fmoe_router_topk(lp.data_ptr(), T, nk, K, _C.F32, scores.data_ptr(), indices.data_ptr(), None, 0, stream())
+        if rc:
+            raise RuntimeError(L.fmoe_last_error().decode())
+
+    ms_fused, ms_topk = event_time_ms(fused, iters), event_time_ms(topk, iters)
+    elt = x.element_size()
+    nbytes = T * H * elt + 2 * nk * H * elt + T * 2 * nk * elt + T * K * (elt + 8)
+    return dict(workload=f"router only: bf16, {T} tokens, hidden {H}, 2x{nk} keys, top-{K}, train-mode batch norm",
+                fused_us=round(ms_fused * 1e3, 2), topk_only_us=round(ms_topk * 1e3, 2),
+                tokens_per_s=round(T / (ms_fused * 1e-3)), algorithmic_bytes=nbytes,
+                achieved_GBps=round(nbytes / (ms_fused * 1e-3) / 1e9, 1), peak_GBps=HBM_PEAK_GBS,
+                gemm_TFLOPs=round(2 * T * H * 2 * nk / (ms_fused * 1e-3) / 1e12, 2))
+
+
+def bench_block_c5(dtype, iters):
+    """The largest single-GPU configuration: 262144 experts of width 2048 (two 1 GiB tables), top-128, renormalised."""
+    import torch
+
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+
+    cfg = C5
+    with torch.device("cuda"):
+        m = FlashMoE(FlashMoEConfig(cfg["hidden"], cfg["inter"], "silu", cfg["experts"], cfg["top_k"], cfg["norm"])).to(dtype)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.normal_(0.0, 0.02, generator=g)
+    x = torch.randn(cfg["batch"], cfg["seq"], cfg["hidden"], device="cuda", generator=g).to(dtype)
+    T = cfg["batch"] * cfg["seq"]
+    with torch.no_grad():
+        ms = event_time_ms(lambda: m(x), iters, warmup=2)
+    return dict(workload=f"C5 full block: bf16, {T} tokens, hidden {cfg['hidden']}, intermediate {cfg['inter']}, "
+                         f"{cfg['experts']} experts, top-{cfg['top_k']}, norm_topk_prob True, train-mode batch norm",
+                ms_per_step=round(ms, 3), tokens_per_s=round(T / (ms * 1e-3)))
+
+
 def cpu_baseline(cfg, dtype, budget_s=20.0):
     """The oracle's block forward on the same workload, on the host cores (checker timed as a baseline)."""
     import torch
@@ -250,6 +319,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-c3", action="store_true")
     ap.add_argument("--only-c3", action="store_true", help="run only the routed-expert kernel on its own shape (for profiling)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the router-only (C2) and largest-block (C5) side measurements")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 256 MiB device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -334,6 +404,14 @@ def main():
         result["expert_c3"] = bench_expert_c3(dtype, max(10, min(50, args.steps)))
         log("expert C3:", result["expert_c3"])
     del keep
+    if not args.no_extras:
+        result["router_c2"] = bench_router_c2(dtype, max(10, min(50, args.steps)))
+        log("router C2:", result["router_c2"])
+        del m, x, fns
+        torch.cuda.empty_cache()
+        result["block_c5"] = bench_block_c5(dtype, 5)
+        log("block C5:", result["block_c5"])
+        torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(C4, dtype)
         log("cpu baseline:", result["cpu_baseline"])

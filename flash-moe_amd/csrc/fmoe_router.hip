@@ -114,9 +114,21 @@ __device__ inline void bitonic_merge_desc(uint64_t (&v)[RK], int lane) {
     for (int j = N >> 1; j >= 1; j >>= 1) bitonic_layer<RK, true>(v, lane, N, j);
 }
 
-// Fold one more group of KP keys into the running sorted-descending top-KP.
-template <int RK, typename Gen>
-__device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_groups, Gen gen) {
+// Key at position `pos` of the wave-wide sequence (wave-uniform `pos`).
+template <int RK>
+__device__ inline uint64_t key_at(const uint64_t (&v)[RK], int pos) {
+    uint64_t k = v[0];
+#pragma unroll
+    for (int r = 1; r < RK; ++r) k = (pos % RK == r) ? v[r] : k;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)k, pos / RK);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(k >> 32), pos / RK);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// Fold groups of KP keys into the running sorted-descending top-KP.  can_stop(g, kth) may end the scan before group
+// g >= 1 when no key of groups g, g+1, ... can exceed `kth`, the key now at position `cut` (the last one kept).
+template <int RK, typename Gen, typename Stop>
+__device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_groups, Gen gen, int cut, Stop can_stop) {
     {
         uint64_t cur[RK];
 #pragma unroll
@@ -126,6 +138,7 @@ __device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_group
         for (int r = 0; r < RK; ++r) best[r] = cur[r];
     }
     for (int g = 1; g < num_groups; ++g) {
+        if (can_stop(g, key_at<RK>(best, cut))) break;
         uint64_t cur[RK];
 #pragma unroll
         for (int r = 0; r < RK; ++r) cur[r] = gen(g, r);
@@ -140,7 +153,7 @@ __device__ inline void topk_groups(uint64_t (&best)[RK], int lane, int num_group
 // output [num_tokens, 2*nk] (both halves of a token side by side) and the per-half log-softmax is computed here, as
 // torch does it: (v - max) - log(sum(exp(v - max))) in fp32; otherwise the input is [2, num_tokens, nk] scores.
 template <typename T, typename TG, int RK, bool FROM_LOGITS>
-__global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
+__global__ __launch_bounds__(kRouterWaves* kWave) __attribute__((amdgpu_waves_per_eu(1, RK >= 4 ? 5 : 8))) void router_topk_kernel(
     const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
     int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets,
     uint32_t row_bytes) {
@@ -149,14 +162,21 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
     __shared__ float half_score[kRouterWaves][2][KP];
     __shared__ uint32_t half_index[kRouterWaves][2][KP];
 
-    // candidate table: all (i, j) with (i+1)*(j+1) <= K, packed i | j << 8
-    for (int i = threadIdx.x; i < top_k; i += blockDim.x) {
-        int off = 0;
-        for (int q = 0; q < i; ++q) off += top_k / (q + 1);
-        const int n = top_k / (i + 1);
-        for (int j = 0; j < n; ++j) cand[off + j] = (uint16_t)(i | (j << 8));
+    // candidate table: all (i, j) with (i+1)*(j+1) <= K, packed i | j << 8, listed by i then j.  Row i has
+    // K/(i+1) entries; the row starts are a running sum over the row lengths (kept in half_index until the table is
+    // built: one division per thread, then additions only).
+    {
+        uint32_t* row_len = &half_index[0][0][0];
+        for (int i = threadIdx.x; i < top_k; i += blockDim.x) row_len[i] = (uint32_t)(top_k / (i + 1));
+        __syncthreads();
+        for (int i = threadIdx.x; i < top_k; i += blockDim.x) {
+            int off = 0;
+            for (int q = 0; q < i; ++q) off += (int)row_len[q];
+            const int n = (int)row_len[i];
+            for (int j = 0; j < n; ++j) cand[off + j] = (uint16_t)(i | (j << 8));
+        }
+        __syncthreads();
     }
-    __syncthreads();
 
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
@@ -188,7 +208,7 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
                     if (p >= nk) return 0ull;
                     const float v = Elem<T>::to_f32(row[p]);
                     return make_key(FROM_LOGITS ? (v - shift) - lse : v, (uint32_t)p);
-                });
+                }, KP - 1, [](int, uint64_t) { return false; });
 #pragma unroll
                 for (int r = 0; r < RK; ++r) {
                     half_score[wave][h][lane * RK + r] = key_score(best[r]);
@@ -207,6 +227,12 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_topk_kernel(
                 const float s = round_through<T>(half_score[wave][0][i] + half_score[wave][1][j]);
                 const uint32_t flat = half_index[wave][0][i] * (uint32_t)nk + half_index[wave][1][j];
                 return make_key(s, flat);
+            }, top_k - 1, [&](int g, uint64_t kth) {
+                // candidates are listed by ascending rank i in half 0, so every sum from group g on is at most
+                // half_score[0][i of the group's first entry] + half_score[1][0]; rounding to T is monotone
+                const int i_first = cand[g * KP] & 0xff;
+                const float bound = round_through<T>(half_score[wave][0][i_first] + half_score[wave][1][0]);
+                return bound < key_score(kth);
             });
             float e[RK];
             float total = 0.0f;

@@ -164,3 +164,52 @@ def test_single_call_block_without_routed_experts():
     y, logits = m(x)
     ref = mlp_forward(x.view(-1, 128), m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight)
     assert torch.equal(y.view(-1, 128), ref) and logits.shape == (2, 64, 32)
+
+
+def test_block_c5_full_size_sampled_tokens():
+    """C5 at full size (32768 tokens, two 1 GiB tables, top-128, normalised gates), evaluation mode so that tokens are
+    independent: the single call equals the staged calls bit for bit, and 48 sampled tokens are checked stage by stage
+    against the oracle (router on the HIP path's fp32 gate output, experts + MLP in float64 on its routing)."""
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+    from flash_moe.ops.hip.flash_block import block_forward
+
+    dtype, T, H, I, E, K, nk = torch.bfloat16, 32768, 2048, 8192, 262144, 128, 512
+    with torch.device("cuda"):
+        m = FlashMoE(FlashMoEConfig(H, I, "silu", E, K, True)).to(dtype)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.normal_(0.0, 0.02, generator=g)
+        m.router_norm.running_mean.normal_(0.0, 0.1, generator=g)
+        m.router_norm.running_var.uniform_(0.5, 1.5, generator=g)
+    m.eval()
+    x = torch.randn(8, 4096, H, device="cuda", generator=g).to(dtype)
+    tokens = x.view(T, H)
+    y, logits, indices, gates = block_forward(tokens, m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight,
+                                              m.router_gate.weight, m.router_norm, m.down_embed.weight, m.up_embed.weight,
+                                              nk, K, True, return_routing=True)
+    assert torch.isfinite(y).all() and torch.isfinite(logits).all()
+    y2, logits2 = m.forward_staged(x)
+    assert torch.equal(y.view_as(y2), y2) and torch.equal(logits.view(T, 2, nk).transpose(0, 1), logits2)
+    assert int(m.router_norm.num_batches_tracked) == 0
+    torch.testing.assert_close(gates.float().sum(-1), torch.ones(T, device="cuda"), rtol=0, atol=2e-2)
+    assert (indices.sort(-1).values.diff(dim=-1) != 0).all() and 0 <= int(indices.min()) and int(indices.max()) < E
+
+    pick = torch.randperm(T, generator=torch.Generator().manual_seed(1))[:48].sort().values.cuda()
+    xs = tokens[pick]
+    _, s_scores, s_idx, s_gates, s_logits32 = m.route(xs, return_logits32=True)
+    assert torch.equal(s_idx, indices[pick]) and torch.equal(s_gates, gates[pick])          # tokens are independent
+    # router: the oracle's exhaustive top-k of the HIP path's own fp32 gate output
+    lp = torch.log_softmax(s_logits32.cpu().view(-1, 2, nk), dim=-1).transpose(0, 1).contiguous()
+    o_s, o_i = orc.router_topk(lp, nk, K + 1)
+    torch.testing.assert_close(s_scores.cpu(), o_s[:, :K], rtol=0, atol=2e-6)
+    set_equal = (s_idx.cpu().sort(-1).values == o_i[:, :K].sort(-1).values).all(-1)
+    assert (set_equal | ((o_s[:, K - 1] - o_s[:, K]).abs() < 2e-6)).all()
+    torch.testing.assert_close(s_gates.float().cpu(), orc.routing_weights(o_s[:, :K], True), rtol=8e-3, atol=1e-10)
+    # experts + MLP in float64 on the sampled tokens, with only the table rows they use
+    rows, remap = torch.unique(s_idx, return_inverse=True)
+    wd_s, wu_s = m.down_embed.weight[rows].cpu().double(), m.up_embed.weight[rows].cpu().double()
+    e64 = orc.expert_forward(xs.cpu().double(), wd_s, wu_s, remap.cpu(), s_gates.cpu().double())
+    y64 = e64 + orc.mlp_forward(xs.cpu().double(), m.gate_proj.weight.cpu().double(), m.up_proj.weight.cpu().double(),
+                                m.down_proj.weight.cpu().double())
+    assert_output_close(y[pick], y64.to(dtype), dtype, "C5 block output vs float64 oracle on sampled tokens")
