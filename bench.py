@@ -284,6 +284,30 @@ def bench_block_c5(dtype, iters):
                 ms_per_step=round(ms, 3), tokens_per_s=round(T / (ms * 1e-3)))
 
 
+def bench_backward_c4(dtype, iters):
+    """Forward + backward of the C4 block through autograd (the differentiable composition of the three ops)."""
+    import torch
+
+    m, x = synthetic_block(C4, dtype, "cuda:0")
+    wy = torch.randn_like(x)
+    T = C4["batch"] * C4["seq"]
+
+    def step():
+        for p in m.parameters():
+            p.grad = None
+        y, _ = m(x.detach().requires_grad_(True))
+        y.backward(wy)
+
+    def forward_only():
+        with torch.no_grad():
+            m.forward_autograd(x)
+
+    ms, ms_fwd = event_time_ms(step, iters, warmup=3), event_time_ms(forward_only, iters, warmup=3)
+    return dict(workload="C4 block, forward + backward through autograd (train-mode batch norm), gradients of the input "
+                         "and of every parameter", ms_per_step=round(ms, 3), tokens_per_s=round(T / (ms * 1e-3)),
+                forward_autograd_ms=round(ms_fwd, 3))
+
+
 def cpu_baseline(cfg, dtype, budget_s=20.0):
     """The oracle's block forward on the same workload, on the host cores (checker timed as a baseline)."""
     import torch
@@ -411,6 +435,9 @@ def main():
         torch.cuda.empty_cache()
         result["block_c5"] = bench_block_c5(dtype, 5)
         log("block C5:", result["block_c5"])
+        torch.cuda.empty_cache()
+        result["backward_c4"] = bench_backward_c4(dtype, 10)
+        log("backward C4:", result["backward_c4"])
         torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(C4, dtype)

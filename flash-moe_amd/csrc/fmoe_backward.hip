@@ -1,0 +1,503 @@
+// Backward passes of the router op, the SwiGLU gate and the routed-expert op for gfx950.
+//
+//   router  : drouter_logits[0,t,i] = sum_{k : idx[t,k] / nk == i} dscores[t,k],  [1,t,j] likewise with idx % nk
+//   swiglu  : c = silu(a) * b  ->  da = dc * (silu(a) * (1 - sigmoid(a)) + sigmoid(a)) * b,  db = dc * silu(a)
+//   experts : out[t] = sum_k silu(s) * g * up[e],  s = <x[t], down[e]>,  e = idx[t,k]:
+//               da_p   = <dout[t], up[e]>                 dg_p = da_p * silu(s)
+//               ds_p   = da_p * g * sigmoid(s) * (1 + s * (1 - sigmoid(s)))
+//               dx[t]  = sum_k ds_p * down[e]
+//               ddown[e] = sum_{p -> e} ds_p * x[t_p]     dup[e] = sum_{p -> e} silu(s_p) * g_p * dout[t_p]
+//
+// Nothing here uses global atomics: every output element is written once, sums run in a fixed order (pairs of an
+// expert in ascending pair index), so gradients are reproducible bit for bit.  The per-token part of the expert
+// backward is one wave per token with the token's rows of x and dout in registers (the layout of the forward
+// row kernel); the per-expert part needs the pairs grouped by expert, which a stable radix sort of (expert, pair)
+// provides (hipCUB, the one library routine in this file), followed by one wave per expert.
+#include <hipcub/hipcub.hpp>
+
+#include "fmoe_common.h"
+#include "fmoe_vec.h"
+
+namespace fmoe {
+namespace {
+
+constexpr int kBwdWaves = 4;
+
+// ------------------------------------------------------------------------------------------------------------
+// router
+// ------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBwdWaves* kWave) void router_backward_kernel(const T* __restrict__ dscores,
+                                                                           const int64_t* __restrict__ indices,
+                                                                           T* __restrict__ dlogits, int64_t num_tokens,
+                                                                           int nk, int top_k, int waves_per_block) {
+    extern __shared__ float acc_all[];   // [waves_per_block][2 * nk], one private row pair per wave
+    const int lane = lane_id();
+    const int wave = (int)(threadIdx.x >> 6);
+    const int64_t token = (int64_t)blockIdx.x * waves_per_block + wave;
+    if (wave >= waves_per_block || token >= num_tokens) return;   // whole waves leave; nobody waits on them
+    float* acc = acc_all + (size_t)wave * 2 * nk;
+    for (int p = lane; p < 2 * nk; p += kWave) acc[p] = 0.0f;
+    __builtin_amdgcn_wave_barrier();
+    const int64_t num_pairs = (int64_t)nk * nk;
+    // LDS adds of one instruction that hit the same address are applied one after the other by the LDS unit, and the
+    // instructions of a wave execute in order, so the sum has a fixed order for given inputs
+    for (int k = lane; k < top_k; k += kWave) {
+        const int64_t id = indices[token * top_k + k];
+        if (id >= 0 && id < num_pairs) {
+            const float d = Elem<T>::to_f32(dscores[token * top_k + k]);
+            __hip_atomic_fetch_add(&acc[(int)(id / nk)], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            __hip_atomic_fetch_add(&acc[nk + (int)(id % nk)], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int p = lane; p < nk; p += kWave) {
+        dlogits[token * nk + p] = Elem<T>::from_f32(acc[p]);
+        dlogits[(num_tokens + token) * nk + p] = Elem<T>::from_f32(acc[nk + p]);
+    }
+}
+
+template <typename T>
+int launch_router_backward(const void* dscores, const int64_t* indices, void* dlogits, int64_t T_, int nk, int K,
+                           hipStream_t stream) {
+    const size_t per_wave = (size_t)2 * nk * sizeof(float);
+    int waves = (int)((48 * 1024) / per_wave);
+    waves = waves < 1 ? 1 : (waves > kBwdWaves ? kBwdWaves : waves);
+    const unsigned grid = (unsigned)((T_ + waves - 1) / waves);
+    hipLaunchKernelGGL((router_backward_kernel<T>), dim3(grid), dim3(kBwdWaves * kWave), waves * per_wave, stream,
+                       (const T*)dscores, indices, (T*)dlogits, T_, nk, K, waves);
+    FMOE_CHECK_LAUNCH("fmoe_router_topk_backward");
+    return FMOE_OK;
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// SwiGLU
+// ------------------------------------------------------------------------------------------------------------
+template <typename T> __device__ inline void unpack16(u32x4_t w, float* v);
+template <> __device__ inline void unpack16<float>(u32x4_t w, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(w[i]);
+}
+template <> __device__ inline void unpack16<bf16_t>(u32x4_t w, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+template <> __device__ inline void unpack16<f16_t>(u32x4_t w, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t wi = w[i];
+        const f16x2_t p = __builtin_bit_cast(f16x2_t, wi);
+        v[2 * i] = (float)p[0];
+        v[2 * i + 1] = (float)p[1];
+    }
+}
+
+// One 16-byte packet per thread.  Row strides (elements) let da / db / h live side by side in wider buffers.
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_backward_kernel(const T* __restrict__ dc, const T* __restrict__ a,
+                                                              const T* __restrict__ b, T* __restrict__ da,
+                                                              T* __restrict__ db, T* __restrict__ h, int64_t rows,
+                                                              int cols, int64_t da_stride, int64_t db_stride) {
+    constexpr int V = Elem<T>::kVec;
+    const int packets = cols / V;
+    const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= rows * packets) return;
+    const int64_t row = q / packets;
+    const int col = (int)(q % packets) * V;
+    const int64_t at = row * cols + col;
+    float dcv[V], av[V], bv[V], dav[V], dbv[V], hv[V];
+    unpack16<T>(*reinterpret_cast<const u32x4_t*>(dc + at), dcv);
+    unpack16<T>(*reinterpret_cast<const u32x4_t*>(a + at), av);
+    unpack16<T>(*reinterpret_cast<const u32x4_t*>(b + at), bv);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const float sig = 1.0f / (1.0f + __expf(-av[v]));
+        const float silu = av[v] * sig;
+        dbv[v] = dcv[v] * silu;
+        dav[v] = dcv[v] * (silu * (1.0f - sig) + sig) * bv[v];
+        hv[v] = silu * bv[v];
+    }
+    *reinterpret_cast<u32x4_t*>(da + row * da_stride + col) = pack16<T>(dav);
+    *reinterpret_cast<u32x4_t*>(db + row * db_stride + col) = pack16<T>(dbv);
+    if (h != nullptr) *reinterpret_cast<u32x4_t*>(h + at) = pack16<T>(hv);
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// routed experts, per-token part: dx, dgates and the two coefficients of every pair
+// ------------------------------------------------------------------------------------------------------------
+template <typename T, int NCH>
+__global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel(
+    const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ down, const T* __restrict__ up,
+    const int64_t* __restrict__ indices, const T* __restrict__ gates, T* __restrict__ dx, T* __restrict__ dgates,
+    float* __restrict__ coef_up, float* __restrict__ coef_down, uint32_t* __restrict__ sort_keys,
+    uint32_t* __restrict__ sort_vals, int64_t num_tokens, int hidden, int64_t num_experts, int top_k) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int PIF = NCH >= 8 ? 1 : (NCH >= 4 ? 2 : 4);   // (down, up) row pairs requested ahead
+    const int lane = lane_id();
+    const int64_t token = (int64_t)blockIdx.x * kBwdWaves + (threadIdx.x >> 6);
+    if (token >= num_tokens) return;
+
+    const int packets = hidden / V;
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    u32x4_t xr[NCH], gr[NCH];
+    bool live[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int p = c * kWave + lane;
+        live[c] = p < packets;
+        xr[c] = live[c] ? reinterpret_cast<const u32x4_t*>(x + token * hidden)[p] : zero4;
+        gr[c] = live[c] ? reinterpret_cast<const u32x4_t*>(dout + token * hidden)[p] : zero4;
+    }
+    float acc[NCH][V];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[c][v] = 0.0f;
+
+    for (int k0 = 0; k0 < top_k; k0 += PIF) {
+        u32x4_t dn[PIF][NCH], uq[PIF][NCH];
+        float gate[PIF];
+        bool valid[PIF];
+        uint32_t expert[PIF];
+#pragma unroll
+        for (int u = 0; u < PIF; ++u) {
+            const int k = k0 + u;
+            int64_t e = -1;
+            gate[u] = 0.0f;
+            if (k < top_k) {
+                e = indices[token * top_k + k];
+                gate[u] = Elem<T>::to_f32(gates[token * top_k + k]);
+            }
+            const uint32_t elo = __builtin_amdgcn_readfirstlane((uint32_t)(e & 0xffffffff));
+            const uint32_t ehi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)e >> 32));
+            e = (int64_t)(((uint64_t)ehi << 32) | elo);
+            valid[u] = e >= 0 && e < num_experts;
+            expert[u] = valid[u] ? (uint32_t)e : (uint32_t)num_experts;
+            const u32x4_t* drow = reinterpret_cast<const u32x4_t*>(down + (valid[u] ? e : 0) * hidden);
+            const u32x4_t* urow = reinterpret_cast<const u32x4_t*>(up + (valid[u] ? e : 0) * hidden);
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const int p = c * kWave + lane;
+                dn[u][c] = (valid[u] && live[c]) ? drow[p] : zero4;
+                uq[u][c] = (valid[u] && live[c]) ? urow[p] : zero4;
+            }
+        }
+        float s[PIF], da[PIF];
+#pragma unroll
+        for (int u = 0; u < PIF; ++u) {
+            float ps = 0.0f, pa = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                ps = dot16<T>(xr[c], dn[u][c], ps);
+                pa = dot16<T>(gr[c], uq[u][c], pa);
+            }
+            s[u] = ps;
+            da[u] = pa;
+        }
+#pragma unroll
+        for (int u = 0; u < PIF; ++u) {
+            s[u] = wave_sum(s[u]);
+            da[u] = wave_sum(da[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < PIF; ++u) {
+            const int k = k0 + u;
+            const float sig = 1.0f / (1.0f + __expf(-s[u]));
+            const float act = s[u] * sig;
+            const float ds = valid[u] ? da[u] * gate[u] * (sig * (1.0f + s[u] * (1.0f - sig))) : 0.0f;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) axpy16<T>(ds, dn[u][c], acc[c]);
+            if (lane == 0 && k < top_k) {
+                const int64_t p = token * top_k + k;
+                coef_up[p] = valid[u] ? act * gate[u] : 0.0f;
+                coef_down[p] = ds;
+                dgates[p] = Elem<T>::from_f32(valid[u] ? da[u] * act : 0.0f);
+                sort_keys[p] = expert[u];
+                sort_vals[p] = (uint32_t)p;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int p = c * kWave + lane;
+        if (live[c]) reinterpret_cast<u32x4_t*>(dx + token * hidden)[p] = pack16<T>(acc[c]);
+    }
+}
+
+// offsets[e] = first position of the sorted key list holding a key >= e, for e in [0, num_experts]
+__global__ __launch_bounds__(256) void expert_offsets_kernel(const uint32_t* __restrict__ keys, int64_t num_pairs,
+                                                             int64_t num_experts, int32_t* __restrict__ offsets) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e > num_experts) return;
+    int64_t lo = 0, hi = num_pairs;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if ((int64_t)keys[mid] < e) lo = mid + 1;
+        else hi = mid;
+    }
+    offsets[e] = (int32_t)lo;
+}
+
+// One wave per expert: its rows of ddown and dup, summed over its pairs in ascending pair index.
+template <typename T, int NCH>
+__global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kernel(
+    const T* __restrict__ dout, const T* __restrict__ x, const float* __restrict__ coef_up,
+    const float* __restrict__ coef_down, const uint32_t* __restrict__ pairs, const int32_t* __restrict__ offsets,
+    T* __restrict__ ddown, T* __restrict__ dup, int hidden, int64_t num_experts, int top_k) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int PIF = NCH >= 8 ? 1 : 2;
+    const int lane = lane_id();
+    const int64_t e = (int64_t)blockIdx.x * kBwdWaves + (threadIdx.x >> 6);
+    if (e >= num_experts) return;
+    const int packets = hidden / V;
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    bool live[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) live[c] = c * kWave + lane < packets;
+    float acc_d[NCH][V], acc_u[NCH][V];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc_d[c][v] = acc_u[c][v] = 0.0f;
+
+    const int begin = offsets[e], end = offsets[e + 1];
+    for (int base = begin; base < end; base += kWave) {
+        const int n = end - base < kWave ? end - base : kWave;
+        // lane j looks up pair base + j: its token and its two coefficients
+        uint32_t tok = 0;
+        float cu = 0.0f, cd = 0.0f;
+        if (lane < n) {
+            const uint32_t p = pairs[base + lane];
+            tok = p / (uint32_t)top_k;
+            cu = coef_up[p];
+            cd = coef_down[p];
+        }
+        for (int j0 = 0; j0 < n; j0 += PIF) {
+            u32x4_t xq[PIF][NCH], gq[PIF][NCH];
+            float su[PIF], sd[PIF];
+#pragma unroll
+            for (int u = 0; u < PIF; ++u) {
+                const int j = j0 + u < n ? j0 + u : n - 1;
+                const bool on = j0 + u < n;
+                const int64_t t = (int64_t)(uint32_t)__builtin_amdgcn_readlane((int)tok, j);
+                su[u] = on ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cu), j)) : 0.0f;
+                sd[u] = on ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cd), j)) : 0.0f;
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    const int p = c * kWave + lane;
+                    xq[u][c] = (on && live[c]) ? reinterpret_cast<const u32x4_t*>(x + t * hidden)[p] : zero4;
+                    gq[u][c] = (on && live[c]) ? reinterpret_cast<const u32x4_t*>(dout + t * hidden)[p] : zero4;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < PIF; ++u)
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    axpy16<T>(sd[u], xq[u][c], acc_d[c]);
+                    axpy16<T>(su[u], gq[u][c], acc_u[c]);
+                }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int p = c * kWave + lane;
+        if (live[c]) {
+            reinterpret_cast<u32x4_t*>(ddown + e * hidden)[p] = pack16<T>(acc_d[c]);
+            reinterpret_cast<u32x4_t*>(dup + e * hidden)[p] = pack16<T>(acc_u[c]);
+        }
+    }
+}
+
+struct ExpertBwdPlan {
+    size_t off_coef_up, off_coef_down, off_keys0, off_keys1, off_vals0, off_vals1, off_offsets, off_sort, sort_bytes, bytes;
+};
+
+ExpertBwdPlan plan_expert_backward(int64_t T_, int64_t E, int K) {
+    ExpertBwdPlan p;
+    const size_t pairs = (size_t)T_ * K;
+    size_t o = 0;
+    auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
+    p.off_coef_up = take(pairs * 4);
+    p.off_coef_down = take(pairs * 4);
+    p.off_keys0 = take(pairs * 4);
+    p.off_keys1 = take(pairs * 4);
+    p.off_vals0 = take(pairs * 4);
+    p.off_vals1 = take(pairs * 4);
+    p.off_offsets = take((size_t)(E + 1) * 4);
+    // scratch of the double-buffered radix sort: block histograms and scan state, measured at ~pairs/16 bytes
+    p.sort_bytes = pairs / 4 + (256u << 10);
+    p.off_sort = take(p.sort_bytes);
+    p.bytes = o;
+    return p;
+}
+
+template <typename T>
+int launch_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,
+                           const void* gates, int64_t T_, int H, int64_t E, int K, void* dx, void* ddown, void* dup,
+                           void* dgates, void* workspace, hipStream_t stream) {
+    constexpr int V = Elem<T>::kVec;
+    const ExpertBwdPlan p = plan_expert_backward(T_, E, K);
+    char* ws = (char*)workspace;
+    float* coef_up = (float*)(ws + p.off_coef_up);
+    float* coef_down = (float*)(ws + p.off_coef_down);
+    uint32_t *keys0 = (uint32_t*)(ws + p.off_keys0), *keys1 = (uint32_t*)(ws + p.off_keys1);
+    uint32_t *vals0 = (uint32_t*)(ws + p.off_vals0), *vals1 = (uint32_t*)(ws + p.off_vals1);
+    int32_t* offsets = (int32_t*)(ws + p.off_offsets);
+    const int64_t pairs = T_ * K;
+    const int nch = (H / V + kWave - 1) / kWave;
+    const dim3 block(kBwdWaves * kWave);
+    const dim3 token_grid((unsigned)((T_ + kBwdWaves - 1) / kBwdWaves));
+    const dim3 expert_grid((unsigned)((E + kBwdWaves - 1) / kBwdWaves));
+
+#define FMOE_LAUNCH_TOKEN(N)                                                                                          \
+    hipLaunchKernelGGL((expert_backward_token_kernel<T, N>), token_grid, block, 0, stream, (const T*)dout, (const T*)x, \
+                       (const T*)down, (const T*)up, indices, (const T*)gates, (T*)dx, (T*)dgates, coef_up, coef_down,  \
+                       keys0, vals0, T_, H, E, K)
+    if (nch <= 1) FMOE_LAUNCH_TOKEN(1);
+    else if (nch <= 2) FMOE_LAUNCH_TOKEN(2);
+    else if (nch <= 4) FMOE_LAUNCH_TOKEN(4);
+    else FMOE_LAUNCH_TOKEN(8);
+#undef FMOE_LAUNCH_TOKEN
+    FMOE_CHECK_LAUNCH("fmoe_expert_backward(tokens)");
+
+    // group the pairs by expert: stable sort of (expert id, pair index); invalid ids carry the key E and sort last
+    int bits = 1;
+    while ((1ll << bits) <= E) ++bits;
+    hipcub::DoubleBuffer<uint32_t> kb(keys0, keys1), vb(vals0, vals1);
+    size_t need = 0;
+    hipError_t err = hipcub::DeviceRadixSort::SortPairs(nullptr, need, kb, vb, (int)pairs, 0, bits, stream);
+    FMOE_REQUIRE(err == hipSuccess, (int)err, "fmoe_expert_backward: sort query failed: %s", hipGetErrorString(err));
+    FMOE_REQUIRE(need <= p.sort_bytes, FMOE_ERR_WORKSPACE, "fmoe_expert_backward: the sort needs %zu bytes of scratch, %zu planned",
+                 need, p.sort_bytes);
+    size_t given = p.sort_bytes;
+    err = hipcub::DeviceRadixSort::SortPairs(ws + p.off_sort, given, kb, vb, (int)pairs, 0, bits, stream);
+    FMOE_REQUIRE(err == hipSuccess, (int)err, "fmoe_expert_backward: sort failed: %s", hipGetErrorString(err));
+    hipLaunchKernelGGL(expert_offsets_kernel, dim3((unsigned)((E + 1 + 255) / 256)), dim3(256), 0, stream, kb.Current(),
+                       pairs, E, offsets);
+    FMOE_CHECK_LAUNCH("fmoe_expert_backward(offsets)");
+
+#define FMOE_LAUNCH_WEIGHT(N)                                                                                            \
+    hipLaunchKernelGGL((expert_backward_weight_kernel<T, N>), expert_grid, block, 0, stream, (const T*)dout, (const T*)x, \
+                       (const float*)coef_up, (const float*)coef_down, (const uint32_t*)vb.Current(),                     \
+                       (const int32_t*)offsets, (T*)ddown, (T*)dup, H, E, K)
+    if (nch <= 1) FMOE_LAUNCH_WEIGHT(1);
+    else if (nch <= 2) FMOE_LAUNCH_WEIGHT(2);
+    else if (nch <= 4) FMOE_LAUNCH_WEIGHT(4);
+    else FMOE_LAUNCH_WEIGHT(8);
+#undef FMOE_LAUNCH_WEIGHT
+    FMOE_CHECK_LAUNCH("fmoe_expert_backward(weights)");
+    return FMOE_OK;
+}
+
+}  // namespace
+
+__global__ void zero_fill_kernel(u32x4_t* __restrict__ p, size_t packets) {
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < packets; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4;
+}
+
+// Used by the MLP backward (fmoe_mlp_backward.hip).
+int launch_swiglu_backward(const void* dc, const void* a, const void* b, void* da, void* db, void* h, int64_t rows, int cols,
+                           int64_t da_stride, int64_t db_stride, int dtype, hipStream_t stream) {
+    const int vec = (int)(16 / dtype_size(dtype));
+    const int64_t packets = rows * (cols / vec);
+    if (packets == 0) return FMOE_OK;
+    const dim3 grid((unsigned)((packets + 255) / 256)), block(256);
+    switch (dtype) {
+        case FMOE_F32:
+            hipLaunchKernelGGL((swiglu_backward_kernel<float>), grid, block, 0, stream, (const float*)dc, (const float*)a,
+                               (const float*)b, (float*)da, (float*)db, (float*)h, rows, cols, da_stride, db_stride);
+            break;
+        case FMOE_BF16:
+            hipLaunchKernelGGL((swiglu_backward_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)dc, (const bf16_t*)a,
+                               (const bf16_t*)b, (bf16_t*)da, (bf16_t*)db, (bf16_t*)h, rows, cols, da_stride, db_stride);
+            break;
+        default:
+            hipLaunchKernelGGL((swiglu_backward_kernel<f16_t>), grid, block, 0, stream, (const f16_t*)dc, (const f16_t*)a,
+                               (const f16_t*)b, (f16_t*)da, (f16_t*)db, (f16_t*)h, rows, cols, da_stride, db_stride);
+    }
+    FMOE_CHECK_LAUNCH("fmoe_swiglu_backward");
+    return FMOE_OK;
+}
+
+}  // namespace fmoe
+
+extern "C" int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64_t num_tokens, int num_keys,
+                                         int top_k, int dtype, void* drouter_logits, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_router_topk_backward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(num_tokens >= 0 && num_keys > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
+                 "fmoe_router_topk_backward: bad shape T=%lld nk=%d K=%d", (long long)num_tokens, num_keys, top_k);
+    FMOE_REQUIRE(num_keys <= 8192, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk_backward: num_keys=%d > 8192", num_keys);
+    if (num_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(drouter_logits && (top_k == 0 || (dscores && indices)), FMOE_ERR_NULL_POINTER,
+                 "fmoe_router_topk_backward: null tensor pointer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FMOE_F32: return launch_router_backward<float>(dscores, indices, drouter_logits, num_tokens, num_keys, top_k, s);
+        case FMOE_BF16: return launch_router_backward<bf16_t>(dscores, indices, drouter_logits, num_tokens, num_keys, top_k, s);
+        default: return launch_router_backward<f16_t>(dscores, indices, drouter_logits, num_tokens, num_keys, top_k, s);
+    }
+}
+
+extern "C" int fmoe_swiglu_backward(const void* dc, const void* a, const void* b, int64_t rows, int cols, int dtype, void* da,
+                                    void* db, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_swiglu_backward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(rows >= 0 && cols > 0, FMOE_ERR_BAD_SHAPE, "fmoe_swiglu_backward: bad shape rows=%lld cols=%d", (long long)rows, cols);
+    if (rows == 0) return FMOE_OK;
+    FMOE_REQUIRE(dc && a && b && da && db, FMOE_ERR_NULL_POINTER, "fmoe_swiglu_backward: null tensor pointer");
+    const int vec = (int)(16 / dtype_size(dtype));
+    FMOE_REQUIRE(cols % vec == 0 && aligned16(dc) && aligned16(a) && aligned16(b) && aligned16(da) && aligned16(db), FMOE_ERR_ALIGNMENT,
+                 "fmoe_swiglu_backward: cols=%d must be a multiple of %d and tensors 16-byte aligned", cols, vec);
+    return launch_swiglu_backward(dc, a, b, da, db, nullptr, rows, cols, cols, cols, dtype, (hipStream_t)stream);
+}
+
+extern "C" size_t fmoe_expert_backward_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
+    if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0 || top_k <= 0 || !fmoe::dtype_ok(dtype)) return 0;
+    return fmoe::plan_expert_backward(num_tokens, num_experts, top_k).bytes;
+}
+
+extern "C" int fmoe_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,
+                                    const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype,
+                                    void* dx, void* ddown, void* dup, void* dgates, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_expert_backward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_experts > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
+                 "fmoe_expert_backward: bad shape T=%lld H=%d E=%lld K=%d", (long long)num_tokens, hidden, (long long)num_experts, top_k);
+    const int vec = (int)(16 / dtype_size(dtype));
+    FMOE_REQUIRE(hidden % vec == 0, FMOE_ERR_ALIGNMENT, "fmoe_expert_backward: hidden=%d must be a multiple of %d (16-byte rows)", hidden, vec);
+    FMOE_REQUIRE(hidden <= 8 * kWave * vec, FMOE_ERR_UNSUPPORTED, "fmoe_expert_backward: hidden=%d exceeds the %d elements per row this build supports",
+                 hidden, 8 * kWave * vec);
+    FMOE_REQUIRE(num_experts < (1ll << 31) - 1 && (int64_t)num_tokens * top_k < (1ll << 31), FMOE_ERR_UNSUPPORTED,
+                 "fmoe_expert_backward: E=%lld or T*K=%lld >= 2^31", (long long)num_experts, (long long)num_tokens * top_k);
+    FMOE_REQUIRE(dx && ddown && dup && x && dout && down && up, FMOE_ERR_NULL_POINTER, "fmoe_expert_backward: null tensor pointer");
+    FMOE_REQUIRE(aligned16(dx) && aligned16(ddown) && aligned16(dup) && aligned16(x) && aligned16(dout) && aligned16(down) && aligned16(up),
+                 FMOE_ERR_ALIGNMENT, "fmoe_expert_backward: tensor pointers must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t elt = dtype_size(dtype);
+    if (num_tokens == 0 || top_k == 0) {   // no pairs: every gradient is zero (a fill kernel, safe under graph capture)
+        const size_t table_packets = (size_t)num_experts * hidden * elt / 16, x_packets = (size_t)num_tokens * hidden * elt / 16;
+        hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, s, (u32x4_t*)ddown, table_packets);
+        hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, s, (u32x4_t*)dup, table_packets);
+        if (x_packets) hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, s, (u32x4_t*)dx, x_packets);
+        FMOE_CHECK_LAUNCH("fmoe_expert_backward(clear)");
+        return FMOE_OK;
+    }
+    FMOE_REQUIRE(indices && gates && dgates, FMOE_ERR_NULL_POINTER, "fmoe_expert_backward: null indices/gates with top_k=%d", top_k);
+    const size_t need = plan_expert_backward(num_tokens, num_experts, top_k).bytes;
+    FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
+                 "fmoe_expert_backward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    switch (dtype) {
+        case FMOE_F32: return launch_expert_backward<float>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dx, ddown, dup, dgates, workspace, s);
+        case FMOE_BF16: return launch_expert_backward<bf16_t>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dx, ddown, dup, dgates, workspace, s);
+        default: return launch_expert_backward<f16_t>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dx, ddown, dup, dgates, workspace, s);
+    }
+}

@@ -10,7 +10,9 @@ pair (:55-105).
   routed experts                                                    ``fmoe_expert_forward``
   shared SwiGLU MLP + add                                           ``fmoe_mlp_forward`` (the add is the second
                                                                     GEMM's epilogue)
-``forward_staged`` runs the same three stages as three calls.
+``forward_staged`` runs the same three stages as three calls.  When gradients are being recorded ``forward`` takes
+``forward_autograd`` instead: the reference's own composition (torch batch norm, linear and log-softmax, then the router,
+expert and MLP ops, flash_moe/modules/flash_moe.py:62-101), whose three ops carry HIP backward passes.
 
 Routing is evaluated in fp32 whatever the module dtype: the normalised activations are rounded to the
 module dtype exactly as the reference does, but their product with the router gate, the log-softmax
@@ -28,9 +30,9 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from flash_moe.ops.hip.flash_block import block_forward
-from flash_moe.ops.hip.flash_expert import expert_forward
-from flash_moe.ops.hip.flash_mlp import mlp_forward
-from flash_moe.ops.hip.flash_router import router_forward
+from flash_moe.ops.hip.flash_expert import expert_forward, flash_expert_func
+from flash_moe.ops.hip.flash_mlp import flash_mlp_func, mlp_forward
+from flash_moe.ops.hip.flash_router import flash_router_func, router_forward
 
 _SILU_NAMES = ("silu", "swish")
 
@@ -86,6 +88,8 @@ class FlashMoE(nn.Module):
         return (router_logits,) + tuple(out[1:])
 
     def forward(self, hidden_states: torch.Tensor, **kwargs):
+        if torch.is_grad_enabled() and (hidden_states.requires_grad or any(p.requires_grad for p in self.parameters())):
+            return self.forward_autograd(hidden_states)
         bsz, seq_len, _ = hidden_states.shape
         tokens = hidden_states.reshape(-1, self.hidden_size)
         out, logits = block_forward(
@@ -93,6 +97,24 @@ class FlashMoE(nn.Module):
             self.router_norm, self.down_embed.weight, self.up_embed.weight, self.num_keys, self.top_k, self.norm_topk_prob,
         )
         router_logits = logits.view(tokens.shape[0], 2, self.num_keys).transpose(0, 1)
+        return out.view(bsz, seq_len, -1), router_logits
+
+    def forward_autograd(self, hidden_states: torch.Tensor):
+        """Differentiable forward.  Routing is evaluated in fp32 as on the fused path: the normalised activations are
+        rounded to the module dtype, their product with the router gate and the log-softmax are fp32."""
+        bsz, seq_len, _ = hidden_states.shape
+        tokens = hidden_states.reshape(-1, self.hidden_size)
+        num_tokens = tokens.shape[0]
+        query = self.router_norm(tokens)
+        logits32 = F.linear(query.float(), self.router_gate.weight.float())
+        router_logits = logits32.to(tokens.dtype).view(num_tokens, 2, self.num_keys).transpose(0, 1)
+        log_probs = F.log_softmax(logits32.view(num_tokens, 2, self.num_keys), dim=-1).transpose(0, 1)
+        scores, indices = flash_router_func(log_probs, self.num_keys, self.top_k)
+        gates = torch.exp(scores)
+        if self.norm_topk_prob:
+            gates = gates / gates.sum(dim=-1, keepdim=True)
+        experts_states = flash_expert_func(tokens, self.down_embed.weight, self.up_embed.weight, indices, gates.to(tokens.dtype))
+        out = flash_mlp_func(tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight) + experts_states
         return out.view(bsz, seq_len, -1), router_logits
 
     def forward_staged(self, hidden_states: torch.Tensor):

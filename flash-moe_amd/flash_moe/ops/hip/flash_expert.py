@@ -47,15 +47,43 @@ def expert_forward(hidden_states, down_weights, up_weights, indices, routing_wei
     return out
 
 
+def expert_backward(dexperts_states, hidden_states, down_weights, up_weights, indices, routing_weights):
+    """Gradients ``(dhidden_states, ddown_weights, dup_weights, drouting_weights)`` of ``expert_forward``
+    (``fmoe_expert_backward``; the reference's _flash_expert_backward, flash_moe/ops/triton/flash_expert.py:654-745).
+    Deterministic; the scores are recomputed rather than saved."""
+    dev = _C.require_gpu(dexperts_states, hidden_states, down_weights, up_weights, indices, routing_weights)
+    do, x, wd, wu, idx, g = (t.contiguous() for t in (dexperts_states, hidden_states, down_weights, up_weights, indices,
+                                                      routing_weights))
+    if do.shape != x.shape or do.dtype != x.dtype:
+        raise ValueError("the output gradient must have the shape and dtype of hidden_states")
+    num_tokens, hidden = x.shape
+    num_experts, top_k = wd.shape[0], idx.shape[1]
+    code = _C.dtype_code(x.dtype)
+    dx, dwd, dwu, dg = torch.empty_like(x), torch.empty_like(wd), torch.empty_like(wu), torch.empty_like(g)
+    L = _C.lib()
+    ws_bytes = L.fmoe_expert_backward_workspace_bytes(num_tokens, hidden, num_experts, top_k, code)
+    ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        status = L.fmoe_expert_backward(
+            _C.ptr(do), _C.ptr(x), _C.ptr(wd), _C.ptr(wu), _C.ptr(idx), _C.ptr(g), num_tokens, hidden, num_experts, top_k,
+            code, _C.ptr(dx), _C.ptr(dwd), _C.ptr(dwu), _C.ptr(dg), _C.ptr(ws), ws_bytes, _C.current_stream(dev),
+        )
+    _C.check(status, "flash_expert backward")
+    return dx, dwd, dwu, dg
+
+
 class FlashExpertFunc(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def forward(ctx, hidden_states, down_weights, up_weights, indices, routing_weights):
+        ctx.save_for_backward(hidden_states, down_weights, up_weights, indices, routing_weights)
         return expert_forward(hidden_states, down_weights, up_weights, indices, routing_weights)
 
     @staticmethod
+    @ensure_contiguous
     def backward(ctx, dexperts_states):
-        raise NotImplementedError("flash_expert backward is not implemented in the HIP path (forward only)")
+        dx, dwd, dwu, dg = expert_backward(dexperts_states, *ctx.saved_tensors)
+        return dx, dwd, dwu, None, dg
 
 
 def flash_expert_func(hidden_states, down_weights, up_weights, indices, routing_weights):

@@ -48,15 +48,59 @@ def mlp_forward(x, gate_weight, up_weight, down_weight, residual: Optional[torch
     return out.view(x.shape)
 
 
+def mlp_backward(dout, x, gate_weight, up_weight, down_weight):
+    """Gradients ``(dx, dgate_weight, dup_weight, ddown_weight)`` of ``mlp_forward`` without residual
+    (``fmoe_mlp_backward``): the gate and up products are recomputed, the SwiGLU gradient is the fused kernel behind
+    ``swiglu_backward``, the transposed-operand GEMMs are rocBLAS calls inside the library."""
+    hidden, inter = x.shape[-1], gate_weight.shape[0]
+    dev = _C.require_gpu(dout, x, gate_weight, up_weight, down_weight)
+    if dout.shape != x.shape or dout.dtype != x.dtype:
+        raise ValueError("the output gradient must have the shape and dtype of x")
+    x2, dy = x.contiguous().view(-1, hidden), dout.contiguous().view(-1, hidden)
+    wg, wu, wd = gate_weight.contiguous(), up_weight.contiguous(), down_weight.contiguous()
+    num_tokens = x2.shape[0]
+    code = _C.dtype_code(x.dtype)
+    dx, dwg, dwu, dwd = torch.empty_like(x2), torch.empty_like(wg), torch.empty_like(wu), torch.empty_like(wd)
+    if num_tokens == 0:
+        return dx.view(x.shape), dwg.zero_(), dwu.zero_(), dwd.zero_()
+    L = _C.lib()
+    ws_bytes = L.fmoe_mlp_backward_workspace_bytes(num_tokens, hidden, inter, code)
+    ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        status = L.fmoe_mlp_backward(
+            _C.ptr(dy), _C.ptr(x2), _C.ptr(wg), _C.ptr(wu), _C.ptr(wd), num_tokens, hidden, inter, code, _C.ptr(dx),
+            _C.ptr(dwg), _C.ptr(dwu), _C.ptr(dwd), _C.ptr(ws), ws_bytes, _C.current_stream(dev),
+        )
+    _C.check(status, "flash_mlp backward")
+    return dx.view(x.shape), dwg, dwu, dwd
+
+
+def swiglu_backward(a: torch.Tensor, b: torch.Tensor, dc: torch.Tensor):
+    """``(da, db)`` for ``c = silu(a) * b`` (``fmoe_swiglu_backward``; flash_moe/ops/triton/flash_mlp.py:126-150)."""
+    if a.shape != b.shape or a.shape != dc.shape or a.dtype != b.dtype or a.dtype != dc.dtype:
+        raise ValueError("a, b and dc must have one shape and dtype")
+    dev = _C.require_gpu(a, b, dc)
+    cols = a.shape[-1]
+    a2, b2, dc2 = (t.contiguous().view(-1, cols) for t in (a, b, dc))
+    da, db = torch.empty_like(a2), torch.empty_like(b2)
+    with torch.cuda.device(dev):
+        status = _C.lib().fmoe_swiglu_backward(_C.ptr(dc2), _C.ptr(a2), _C.ptr(b2), a2.shape[0], cols, _C.dtype_code(a.dtype),
+                                               _C.ptr(da), _C.ptr(db), _C.current_stream(dev))
+    _C.check(status, "swiglu backward")
+    return da.view(a.shape), db.view(a.shape)
+
+
 class FlashMLPFunc(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def forward(ctx, x, gate_weight, up_weight, down_weight):
+        ctx.save_for_backward(x, gate_weight, up_weight, down_weight)
         return mlp_forward(x, gate_weight, up_weight, down_weight)
 
     @staticmethod
+    @ensure_contiguous
     def backward(ctx, dout):
-        raise NotImplementedError("flash_mlp backward is not implemented in the HIP path (forward only)")
+        return mlp_backward(dout, *ctx.saved_tensors)
 
 
 def flash_mlp_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor, down_weight: torch.Tensor) -> torch.Tensor:

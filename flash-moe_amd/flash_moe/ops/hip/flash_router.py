@@ -109,6 +109,21 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
     return logits, scores, indices, gates
 
 
+def router_topk_backward(dscores: torch.Tensor, indices: torch.Tensor, num_expert_keys: int) -> torch.Tensor:
+    """Scatter of ``dscores`` [T, K] onto the two halves' keys -> [2, T, nk] in ``dscores.dtype`` (``fmoe_router_topk_backward``)."""
+    if dscores.dim() != 2 or indices.shape != dscores.shape or indices.dtype != torch.int64:
+        raise ValueError("expected dscores [T, K] and int64 indices of the same shape")
+    dev = _C.require_gpu(dscores, indices)
+    ds, idx = dscores.contiguous(), indices.contiguous()
+    T, K = ds.shape
+    out = torch.empty((2, T, num_expert_keys), device=dev, dtype=ds.dtype)
+    with torch.cuda.device(dev):
+        status = _C.lib().fmoe_router_topk_backward(_C.ptr(ds), _C.ptr(idx), T, num_expert_keys, K, _C.dtype_code(ds.dtype),
+                                                    _C.ptr(out), _C.current_stream(dev))
+    _C.check(status, "flash_router backward")
+    return out
+
+
 class FlashRouterFunc(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
@@ -116,11 +131,17 @@ class FlashRouterFunc(torch.autograd.Function):
         """router_logits [2, T, nk] -> scores [T, K] (dtype of the input), indices [T, K] int64."""
         scores, indices, _ = router_topk_gates(router_logits, num_expert_keys, num_experts_per_tok)
         ctx.mark_non_differentiable(indices)
+        ctx.save_for_backward(indices)
+        ctx.num_expert_keys = num_expert_keys
         return scores, indices
 
     @staticmethod
+    @ensure_contiguous
     def backward(ctx, dscores, dindices):
-        raise NotImplementedError("flash_router backward is not implemented in the HIP path (forward only)")
+        """drouter_logits [2, T, nk]: each selected pair's gradient goes to its two keys
+        (flash_moe/ops/triton/flash_router.py:317-344); no gradient for the two integers."""
+        (indices,) = ctx.saved_tensors
+        return router_topk_backward(dscores, indices, ctx.num_expert_keys), None, None
 
 
 def flash_router_func(router_logits, num_expert_keys, num_experts_per_tok):

@@ -38,7 +38,8 @@ typedef enum {
     FMOE_ERR_BAD_DTYPE = -4,      /* dtype not one of fmoe_dtype_t */
     FMOE_ERR_UNSUPPORTED = -5,    /* extent beyond what the kernels are built for (message says which) */
     FMOE_ERR_ALIGNMENT = -6,      /* pointer not 16-byte aligned or row length not a multiple of 16 bytes */
-    FMOE_ERR_WORKSPACE = -7       /* workspace NULL or smaller than the *_workspace_bytes() figure */
+    FMOE_ERR_WORKSPACE = -7,      /* workspace NULL or smaller than the *_workspace_bytes() figure */
+    FMOE_ERR_LIBRARY = -8         /* rocBLAS (backward GEMMs only) could not be loaded or reported a failure */
 } fmoe_status_t;
 
 /* ABI version of the loaded library (== FMOE_ABI_VERSION it was built with). */
@@ -178,6 +179,42 @@ int fmoe_block_forward(const void* x, const void* gate_proj_w, const void* up_pr
                        float eps, int64_t num_tokens, int hidden, int intermediate, int64_t num_experts, int num_keys,
                        int top_k, int dtype, int norm_topk_prob, void* out, void* router_logits, int64_t* indices_out,
                        void* gates_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ================================================================================================
+ * Backward passes.  Deterministic: no global atomics, every gradient element is written once.
+ * ================================================================================================ */
+
+/* FlashRouterFunc.backward / _flash_router_backward / _bwd_kernel (flash_moe/ops/triton/flash_router.py:317-344,
+ * 205-249): drouter_logits [2, T, nk] (dtype), fully written:
+ *   [0,t,i] = sum of dscores[t,k] over k with indices[t,k] / nk == i;  [1,t,j] likewise with indices[t,k] % nk.
+ * dscores [T, K] dtype, indices [T, K] int64 (ids outside [0, nk*nk) contribute nothing).  num_keys <= 8192. */
+int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64_t num_tokens, int num_keys, int top_k,
+                              int dtype, void* drouter_logits, void* stream);
+
+/* swiglu_backward / _swiglu_backward_kernel (flash_moe/ops/triton/flash_mlp.py:64-102, 126-150): for c = silu(a) * b,
+ *   da = dc * (silu(a) * (1 - sigmoid(a)) + sigmoid(a)) * b,   db = dc * silu(a),   all [rows, cols] dtype. */
+int fmoe_swiglu_backward(const void* dc, const void* a, const void* b, int64_t rows, int cols, int dtype, void* da,
+                         void* db, void* stream);
+
+/* Backward of triton_flash_mlp_func (flash_moe/ops/triton/flash_mlp.py:169-181: two matmuls, TritonSwiGLUFunc, one
+ * matmul, differentiated by autograd in the reference): from dy [T,H] the gradients dx [T,H], dgate_w, dup_w [I,H],
+ * ddown_w [H,I].  The gate and up products are recomputed; the transposed-operand GEMMs are rocBLAS calls (loaded on
+ * first use; FMOE_ERR_LIBRARY if unavailable). */
+size_t fmoe_mlp_backward_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int dtype);
+
+int fmoe_mlp_backward(const void* dy, const void* x, const void* gate_w, const void* up_w, const void* down_w,
+                      int64_t num_tokens, int hidden, int intermediate, int dtype, void* dx, void* dgate_w, void* dup_w,
+                      void* ddown_w, void* workspace, size_t workspace_bytes, void* stream);
+
+/* FlashExpertFunc.backward / _flash_expert_backward (flash_moe/ops/triton/flash_expert.py:654-745, kernels :234-525):
+ * from dout [T,H] the gradients dx [T,H], ddown, dup [E,H] (rows of experts no pair selects are zero) and
+ * dgates [T,K]; indices get none.  Scores are recomputed, not saved.  Requires T*K < 2^31. */
+size_t fmoe_expert_backward_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
+
+int fmoe_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,
+                         const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype,
+                         void* dx, void* ddown, void* dup, void* dgates, void* workspace, size_t workspace_bytes,
+                         void* stream);
 
 #ifdef __cplusplus
 }

@@ -140,6 +140,48 @@ def test_block_argument_checks():
     assert call(T=0, x=None, ws=None, ws_bytes=0) == 0
 
 
+def test_backward_argument_checks():
+    lib = _C.lib()
+    keep, a = _buf()
+    rb = lib.fmoe_router_topk_backward
+    assert rb(a, a, 4, 8, 2, 9, a, None) == -4
+    assert rb(a, a, 4, 0, 2, _C.F32, a, None) == -2
+    assert rb(a, a, 4, 9000, 2, _C.F32, a, None) == -5
+    assert rb(a, None, 4, 8, 2, _C.F32, a, None) == -1
+    assert rb(None, None, 0, 8, 2, _C.F32, None, None) == 0
+    sb = lib.fmoe_swiglu_backward
+    assert sb(a, a, a, 4, 64, 7, a, a, None) == -4
+    assert sb(a, a, a, 4, 0, _C.BF16, a, a, None) == -2
+    assert sb(a, a, a, 4, 60, _C.BF16, a, a, None) == -6
+    assert sb(a, None, a, 4, 64, _C.BF16, a, a, None) == -1
+    assert sb(None, None, None, 0, 64, _C.BF16, None, None, None) == 0
+    need = lib.fmoe_expert_backward_workspace_bytes(8, 64, 256, 4, _C.BF16)
+    assert need >= 8 * 4 * 24 + 257 * 4 and need % 256 == 0
+    eb = lib.fmoe_expert_backward
+
+    def ecall(T=8, H=64, E=256, K=4, dtype=_C.BF16, dout=a, ws=a, ws_bytes=need):
+        return eb(dout, a, a, a, a, a, T, H, E, K, dtype, a, a, a, a, ws, ws_bytes, None)
+
+    assert ecall(dtype=3) == -4
+    assert ecall(H=0) == -2
+    assert ecall(H=60) == -6
+    assert ecall(H=8192) == -5
+    assert ecall(dout=None) == -1
+    assert ecall(ws_bytes=need - 1) == -7
+    mneed = lib.fmoe_mlp_backward_workspace_bytes(8, 64, 128, _C.BF16)
+    assert mneed >= 6 * 8 * 128 * 2 and mneed % 256 == 0
+    mb = lib.fmoe_mlp_backward
+
+    def mcall(T=8, H=64, I=128, dtype=_C.BF16, dy=a, ws_bytes=mneed):
+        return mb(dy, a, a, a, a, T, H, I, dtype, a, a, a, a, a, ws_bytes, None)
+
+    assert mcall(dtype=5) == -4
+    assert mcall(T=0) == -2
+    assert mcall(I=100) == -6
+    assert mcall(dy=None) == -1
+    assert mcall(ws_bytes=mneed - 1) == -7
+
+
 def test_python_wrappers_refuse_cpu_tensors():
     from flash_moe.ops import flash_expert_func, flash_mlp_func, flash_router_func
 

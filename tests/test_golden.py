@@ -103,8 +103,15 @@ def _hip_block(H, I, E, K, norm, w, dtype=torch.float32):
     return m.to(device="cuda", dtype=dtype)
 
 
+@pytest.fixture
+def fused_forward_path():
+    """The module takes its fused forward when no gradient is being recorded."""
+    with torch.no_grad():
+        yield
+
+
 @pytest.mark.gpu
-def test_hip_block_reproduces_small_block():
+def test_hip_block_reproduces_small_block(fused_forward_path):
     g = load("block_small_fp32.npz")
     x = torch.from_numpy(g["x"])
     w = small_weights(g)
@@ -129,7 +136,7 @@ def test_hip_block_reproduces_small_block():
 
 
 @pytest.mark.gpu
-def test_hip_block_reproduces_c1():
+def test_hip_block_reproduces_c1(fused_forward_path):
     g = load("block_c1_fp32.npz")
     x, w = make_golden.c1_inputs()
     m = _hip_block(256, 1024, 1024, 16, False, w)
