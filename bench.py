@@ -343,6 +343,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-c3", action="store_true")
     ap.add_argument("--only-c3", action="store_true", help="run only the routed-expert kernel on its own shape (for profiling)")
+    ap.add_argument("--only-backward", action="store_true", help="run only forward + backward of the C4 block (for profiling)")
     ap.add_argument("--no-extras", action="store_true", help="skip the router-only (C2) and largest-block (C5) side measurements")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 256 MiB device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
@@ -374,6 +375,13 @@ def main():
         log("expert C3:", res)
         print(json.dumps({"metric": "expert kernel HBM GB/s", "value": res["achieved_GBps"], "unit": "GB/s", "n_gpus": 1,
                           "steps": args.steps, "warmup": args.warmup, "expert_c3": res}), flush=True)
+        return
+    if args.only_backward:
+        res = bench_backward_c4(dtype, max(5, min(20, args.steps)))
+        log("backward C4:", res)
+        print(json.dumps({"metric": "FlashMoE fwd+bwd tokens/s (h1024, 16K experts, top-64)", "value": res["tokens_per_s"],
+                          "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "backward_c4": res}),
+              flush=True)
         return
     m, x = synthetic_block(C4, dtype, "cuda:0")
     T = C4["batch"] * C4["seq"]
