@@ -8,13 +8,12 @@
 //               dx[t]  = sum_k ds_p * down[e]
 //               ddown[e] = sum_{p -> e} ds_p * x[t_p]     dup[e] = sum_{p -> e} silu(s_p) * g_p * dout[t_p]
 //
-// Nothing here uses global atomics: every output element is written once, sums run in a fixed order (pairs of an
-// expert in ascending pair index), so gradients are reproducible bit for bit.  The per-token part of the expert
-// backward is one wave per token with the token's rows of x and dout in registers (the layout of the forward
-// row kernel); the per-expert part needs the pairs grouped by expert, which a stable radix sort of (expert, pair)
-// provides (hipCUB, the one library routine in this file), followed by one wave per expert.
-#include <hipcub/hipcub.hpp>
-
+// No floating-point atomics on global memory: every output element is written once and sums run in a fixed order
+// (pairs of an expert in ascending pair index), so gradients are reproducible bit for bit.  The per-token part of the
+// expert backward is one wave per token with the token's rows of x and dout in registers (the layout of the forward
+// row kernel).  The per-expert part needs the pairs grouped by expert: a counting sort (integer histogram, exclusive
+// scan, fill through per-expert cursors) puts each expert's pairs in one segment in arbitrary order, and the wave that
+// owns the expert walks its segment in ascending pair index by repeatedly taking the smallest index not yet used.
 #include "fmoe_common.h"
 #include "fmoe_vec.h"
 
@@ -132,8 +131,8 @@ template <typename T, int NCH>
 __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel(
     const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ down, const T* __restrict__ up,
     const int64_t* __restrict__ indices, const T* __restrict__ gates, T* __restrict__ dx, T* __restrict__ dgates,
-    float* __restrict__ coef_up, float* __restrict__ coef_down, uint32_t* __restrict__ sort_keys,
-    uint32_t* __restrict__ sort_vals, int64_t num_tokens, int hidden, int64_t num_experts, int top_k) {
+    float* __restrict__ coef_up, float* __restrict__ coef_down, int32_t* __restrict__ counts, int64_t num_tokens,
+    int hidden, int64_t num_experts, int top_k) {
     constexpr int V = Elem<T>::kVec;
     constexpr int PIF = NCH >= 8 ? 1 : (NCH >= 4 ? 2 : 4);   // (down, up) row pairs requested ahead
     const int lane = lane_id();
@@ -161,7 +160,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel
         u32x4_t dn[PIF][NCH], uq[PIF][NCH];
         float gate[PIF];
         bool valid[PIF];
-        uint32_t expert[PIF];
+        int64_t expert[PIF];
 #pragma unroll
         for (int u = 0; u < PIF; ++u) {
             const int k = k0 + u;
@@ -175,7 +174,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel
             const uint32_t ehi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)e >> 32));
             e = (int64_t)(((uint64_t)ehi << 32) | elo);
             valid[u] = e >= 0 && e < num_experts;
-            expert[u] = valid[u] ? (uint32_t)e : (uint32_t)num_experts;
+            expert[u] = e;
             const u32x4_t* drow = reinterpret_cast<const u32x4_t*>(down + (valid[u] ? e : 0) * hidden);
             const u32x4_t* urow = reinterpret_cast<const u32x4_t*>(up + (valid[u] ? e : 0) * hidden);
 #pragma unroll
@@ -215,8 +214,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel
                 coef_up[p] = valid[u] ? act * gate[u] : 0.0f;
                 coef_down[p] = ds;
                 dgates[p] = Elem<T>::from_f32(valid[u] ? da[u] * act : 0.0f);
-                sort_keys[p] = expert[u];
-                sort_vals[p] = (uint32_t)p;
+                if (valid[u]) atomicAdd(&counts[expert[u]], 1);   // integer histogram: the result does not depend on order
             }
         }
     }
@@ -227,18 +225,48 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel
     }
 }
 
-// offsets[e] = first position of the sorted key list holding a key >= e, for e in [0, num_experts]
-__global__ __launch_bounds__(256) void expert_offsets_kernel(const uint32_t* __restrict__ keys, int64_t num_pairs,
-                                                             int64_t num_experts, int32_t* __restrict__ offsets) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e > num_experts) return;
-    int64_t lo = 0, hi = num_pairs;
-    while (lo < hi) {
-        const int64_t mid = (lo + hi) >> 1;
-        if ((int64_t)keys[mid] < e) lo = mid + 1;
-        else hi = mid;
+__global__ void zero_i32_kernel(int32_t* __restrict__ p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+// offsets[e] = number of pairs of experts < e, for e in [0, num_experts]; one workgroup, each thread owns a run of experts.
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void expert_scan_kernel(const int32_t* __restrict__ counts,
+                                                                  int32_t* __restrict__ offsets, int64_t num_experts) {
+    __shared__ int32_t wave_total[kScanThreads / kWave];
+    const int tid = (int)threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int64_t per = (num_experts + kScanThreads - 1) / kScanThreads;
+    const int64_t lo = (int64_t)tid * per, hi = lo + per < num_experts ? lo + per : num_experts;
+    int32_t mine = 0;
+    for (int64_t e = lo; e < hi; ++e) mine += counts[e];
+    // inclusive scan over the wave, then over the wave totals
+    int32_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += up;
     }
-    offsets[e] = (int32_t)lo;
+    if (lane == kWave - 1) wave_total[wave] = incl;
+    __syncthreads();
+    int32_t before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_total[w];
+    int32_t run = before + incl - mine;
+    for (int64_t e = lo; e < hi; ++e) {
+        offsets[e] = run;
+        run += counts[e];
+    }
+    if (tid == kScanThreads - 1) offsets[num_experts] = before + incl;
+}
+
+// pairs[offsets[e] + (arrival order)] = p for every valid pair: segments are complete, their internal order is not fixed
+__global__ __launch_bounds__(256) void expert_fill_kernel(const int64_t* __restrict__ indices, const int32_t* __restrict__ offsets,
+                                                          int32_t* __restrict__ cursor, uint32_t* __restrict__ pairs,
+                                                          int64_t num_pairs, int64_t num_experts) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= num_pairs) return;
+    const int64_t e = indices[p];
+    if (e < 0 || e >= num_experts) return;
+    pairs[offsets[e] + atomicAdd(&cursor[e], 1)] = (uint32_t)p;
 }
 
 // One wave per expert: its rows of ddown and dup, summed over its pairs in ascending pair index.
@@ -264,16 +292,46 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
         for (int v = 0; v < V; ++v) acc_d[c][v] = acc_u[c][v] = 0.0f;
 
     const int begin = offsets[e], end = offsets[e + 1];
-    for (int base = begin; base < end; base += kWave) {
-        const int n = end - base < kWave ? end - base : kWave;
-        // lane j looks up pair base + j: its token and its two coefficients
+    const int n_total = end - begin;
+    // The segment is walked in ascending pair index, kWave pairs per round: the round takes the kWave smallest indices
+    // above the last one used.  Segments of at most kWave pairs (the usual case) are read once.
+    uint32_t floor_excl = 0;     // pairs with index < floor_excl are done (pair indices are distinct)
+    for (int done = 0; done < n_total; done += kWave) {
+        const int n = n_total - done < kWave ? n_total - done : kWave;
+        uint32_t mine = 0xFFFFFFFFu;   // this lane's pair of the round: the (lane)-th smallest index >= floor_excl
+        if (n_total <= kWave) {
+            // rank of each pair inside the segment by counting smaller ones
+            const uint32_t p = lane < n_total ? pairs[begin + lane] : 0xFFFFFFFFu;
+            int rank = 0;
+            for (int j = 0; j < n_total; ++j) rank += ((uint32_t)__builtin_amdgcn_readlane((int)p, j) < p) ? 1 : 0;
+            // lane `rank` takes p: a permutation of the live lanes
+            const int got = __builtin_amdgcn_ds_permute(rank << 2, (int)p);
+            mine = lane < n_total ? (uint32_t)got : 0xFFFFFFFFu;
+        } else {
+            // long segment: kWave selection passes over it, each taking the smallest remaining index
+            uint32_t last = floor_excl;
+            for (int r = 0; r < n; ++r) {
+                uint32_t best = 0xFFFFFFFFu;
+                for (int j = lane; j < n_total; j += kWave) {
+                    const uint32_t p = pairs[begin + j];
+                    if (p >= last && p < best) best = p;
+                }
+#pragma unroll
+                for (int d = 32; d >= 1; d >>= 1) {
+                    const uint32_t o = (uint32_t)__shfl_xor((int)best, d, kWave);
+                    best = o < best ? o : best;
+                }
+                if (lane == r) mine = best;
+                last = best + 1;
+            }
+            floor_excl = last;
+        }
         uint32_t tok = 0;
         float cu = 0.0f, cd = 0.0f;
         if (lane < n) {
-            const uint32_t p = pairs[base + lane];
-            tok = p / (uint32_t)top_k;
-            cu = coef_up[p];
-            cd = coef_down[p];
+            tok = mine / (uint32_t)top_k;
+            cu = coef_up[mine];
+            cd = coef_down[mine];
         }
         for (int j0 = 0; j0 < n; j0 += PIF) {
             u32x4_t xq[PIF][NCH], gq[PIF][NCH];
@@ -312,7 +370,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
 }
 
 struct ExpertBwdPlan {
-    size_t off_coef_up, off_coef_down, off_keys0, off_keys1, off_vals0, off_vals1, off_offsets, off_sort, sort_bytes, bytes;
+    size_t off_coef_up, off_coef_down, off_pairs, off_counts, off_cursor, off_offsets, bytes;
 };
 
 ExpertBwdPlan plan_expert_backward(int64_t T_, int64_t E, int K) {
@@ -322,14 +380,10 @@ ExpertBwdPlan plan_expert_backward(int64_t T_, int64_t E, int K) {
     auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
     p.off_coef_up = take(pairs * 4);
     p.off_coef_down = take(pairs * 4);
-    p.off_keys0 = take(pairs * 4);
-    p.off_keys1 = take(pairs * 4);
-    p.off_vals0 = take(pairs * 4);
-    p.off_vals1 = take(pairs * 4);
+    p.off_pairs = take(pairs * 4);
+    p.off_counts = take((size_t)E * 4);        // counts and cursor are adjacent: one clearing launch
+    p.off_cursor = take((size_t)E * 4);
     p.off_offsets = take((size_t)(E + 1) * 4);
-    // scratch of the double-buffered radix sort: block histograms and scan state, measured at ~pairs/16 bytes
-    p.sort_bytes = pairs / 4 + (256u << 10);
-    p.off_sort = take(p.sort_bytes);
     p.bytes = o;
     return p;
 }
@@ -343,8 +397,9 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
     char* ws = (char*)workspace;
     float* coef_up = (float*)(ws + p.off_coef_up);
     float* coef_down = (float*)(ws + p.off_coef_down);
-    uint32_t *keys0 = (uint32_t*)(ws + p.off_keys0), *keys1 = (uint32_t*)(ws + p.off_keys1);
-    uint32_t *vals0 = (uint32_t*)(ws + p.off_vals0), *vals1 = (uint32_t*)(ws + p.off_vals1);
+    uint32_t* pairs_by_expert = (uint32_t*)(ws + p.off_pairs);
+    int32_t* counts = (int32_t*)(ws + p.off_counts);
+    int32_t* cursor = (int32_t*)(ws + p.off_cursor);
     int32_t* offsets = (int32_t*)(ws + p.off_offsets);
     const int64_t pairs = T_ * K;
     const int nch = (H / V + kWave - 1) / kWave;
@@ -352,10 +407,13 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
     const dim3 token_grid((unsigned)((T_ + kBwdWaves - 1) / kBwdWaves));
     const dim3 expert_grid((unsigned)((E + kBwdWaves - 1) / kBwdWaves));
 
+    const int64_t clear = (int64_t)((p.off_cursor - p.off_counts) / 4) + E;
+    hipLaunchKernelGGL(zero_i32_kernel, dim3(256), dim3(256), 0, stream, counts, clear);
+    FMOE_CHECK_LAUNCH("fmoe_expert_backward(clear)");
 #define FMOE_LAUNCH_TOKEN(N)                                                                                          \
     hipLaunchKernelGGL((expert_backward_token_kernel<T, N>), token_grid, block, 0, stream, (const T*)dout, (const T*)x, \
                        (const T*)down, (const T*)up, indices, (const T*)gates, (T*)dx, (T*)dgates, coef_up, coef_down,  \
-                       keys0, vals0, T_, H, E, K)
+                       counts, T_, H, E, K)
     if (nch <= 1) FMOE_LAUNCH_TOKEN(1);
     else if (nch <= 2) FMOE_LAUNCH_TOKEN(2);
     else if (nch <= 4) FMOE_LAUNCH_TOKEN(4);
@@ -363,25 +421,15 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
 #undef FMOE_LAUNCH_TOKEN
     FMOE_CHECK_LAUNCH("fmoe_expert_backward(tokens)");
 
-    // group the pairs by expert: stable sort of (expert id, pair index); invalid ids carry the key E and sort last
-    int bits = 1;
-    while ((1ll << bits) <= E) ++bits;
-    hipcub::DoubleBuffer<uint32_t> kb(keys0, keys1), vb(vals0, vals1);
-    size_t need = 0;
-    hipError_t err = hipcub::DeviceRadixSort::SortPairs(nullptr, need, kb, vb, (int)pairs, 0, bits, stream);
-    FMOE_REQUIRE(err == hipSuccess, (int)err, "fmoe_expert_backward: sort query failed: %s", hipGetErrorString(err));
-    FMOE_REQUIRE(need <= p.sort_bytes, FMOE_ERR_WORKSPACE, "fmoe_expert_backward: the sort needs %zu bytes of scratch, %zu planned",
-                 need, p.sort_bytes);
-    size_t given = p.sort_bytes;
-    err = hipcub::DeviceRadixSort::SortPairs(ws + p.off_sort, given, kb, vb, (int)pairs, 0, bits, stream);
-    FMOE_REQUIRE(err == hipSuccess, (int)err, "fmoe_expert_backward: sort failed: %s", hipGetErrorString(err));
-    hipLaunchKernelGGL(expert_offsets_kernel, dim3((unsigned)((E + 1 + 255) / 256)), dim3(256), 0, stream, kb.Current(),
-                       pairs, E, offsets);
-    FMOE_CHECK_LAUNCH("fmoe_expert_backward(offsets)");
+    hipLaunchKernelGGL(expert_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, (const int32_t*)counts, offsets, E);
+    FMOE_CHECK_LAUNCH("fmoe_expert_backward(scan)");
+    hipLaunchKernelGGL(expert_fill_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, indices,
+                       (const int32_t*)offsets, cursor, pairs_by_expert, pairs, E);
+    FMOE_CHECK_LAUNCH("fmoe_expert_backward(fill)");
 
 #define FMOE_LAUNCH_WEIGHT(N)                                                                                            \
     hipLaunchKernelGGL((expert_backward_weight_kernel<T, N>), expert_grid, block, 0, stream, (const T*)dout, (const T*)x, \
-                       (const float*)coef_up, (const float*)coef_down, (const uint32_t*)vb.Current(),                     \
+                       (const float*)coef_up, (const float*)coef_down, (const uint32_t*)pairs_by_expert,                  \
                        (const int32_t*)offsets, (T*)ddown, (T*)dup, H, E, K)
     if (nch <= 1) FMOE_LAUNCH_WEIGHT(1);
     else if (nch <= 2) FMOE_LAUNCH_WEIGHT(2);
