@@ -14,11 +14,20 @@
 namespace fmoe {
 namespace {
 
+// What is applied to the score <x, down[e]> before the gate: the routed experts of FlashMoE use SiLU, PEER uses the
+// erf GELU, and a product-key memory has no score at all (its coefficient is the routing weight itself).
+enum Activation { kActSilu = 0, kActGelu = 1, kActNone = 2 };
+template <int ACT> __device__ inline float activate(float s) {
+    if (ACT == kActSilu) return silu_f32(s);
+    if (ACT == kActGelu) return 0.5f * s * (1.0f + erff(s * 0.70710678118654752440f));
+    return 1.0f;
+}
+
 constexpr int kPairsInFlight = 4;   // (down,up) row pairs requested ahead per wave
 constexpr int kWavesPerBlock = 4;
 
 // NCH = number of 16-byte packets each lane holds per row: a row has at most NCH*64 packets.
-template <typename T, int NCH>
+template <typename T, int NCH, int ACT>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
     const T* __restrict__ x, const T* __restrict__ down, const T* __restrict__ up,
     const int64_t* __restrict__ indices, const T* __restrict__ gates, T* __restrict__ out,
@@ -37,7 +46,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
     for (int c = 0; c < NCH; ++c) {
         const int p = c * kWave + lane;
         live[c] = p < packets;
-        xr[c] = live[c] ? reinterpret_cast<const u32x4_t*>(x + token * hidden)[p] : zero4;
+        xr[c] = (ACT != kActNone && live[c]) ? reinterpret_cast<const u32x4_t*>(x + token * hidden)[p] : zero4;
     }
 
     float acc[NCH][V];
@@ -73,7 +82,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
                 const int p = c * kWave + lane;
-                dn[u][c] = (ok && live[c]) ? drow[p] : zero4;
+                dn[u][c] = (ACT != kActNone && ok && live[c]) ? drow[p] : zero4;
                 uq[u][c] = (ok && live[c]) ? urow[p] : zero4;
             }
         }
@@ -85,11 +94,13 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
             for (int c = 0; c < NCH; ++c) part = dot16<T>(xr[c], dn[u][c], part);
             s[u] = part;
         }
+        if (ACT != kActNone) {
 #pragma unroll
-        for (int u = 0; u < kPairsInFlight; ++u) s[u] = wave_sum(s[u]);
+            for (int u = 0; u < kPairsInFlight; ++u) s[u] = wave_sum(s[u]);
+        }
 #pragma unroll
         for (int u = 0; u < kPairsInFlight; ++u) {
-            const float a = silu_f32(s[u]) * gate[u];
+            const float a = activate<ACT>(s[u]) * gate[u];
 #pragma unroll
             for (int c = 0; c < NCH; ++c) axpy16<T>(a, uq[u][c], acc[c]);
         }
@@ -103,16 +114,22 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
 }
 
 template <typename T>
-int launch_expert_rows(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
-                  int64_t T_, int H, int64_t E, int K, void* out, hipStream_t stream) {
+int launch_expert_rows(int act, const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
+                       int64_t T_, int H, int64_t E, int K, void* out, hipStream_t stream) {
     constexpr int V = Elem<T>::kVec;
     const int packets = H / V;
     const int nch = (packets + kWave - 1) / kWave;
     const dim3 block(kWavesPerBlock * kWave);
     const dim3 grid((unsigned)((T_ + kWavesPerBlock - 1) / kWavesPerBlock));
-#define FMOE_LAUNCH_EXPERT(N)                                                                            \
-    hipLaunchKernelGGL((expert_token_kernel<T, N>), grid, block, 0, stream, (const T*)x, (const T*)down, \
+#define FMOE_LAUNCH_EXPERT_ACT(N, A)                                                                        \
+    hipLaunchKernelGGL((expert_token_kernel<T, N, A>), grid, block, 0, stream, (const T*)x, (const T*)down, \
                        (const T*)up, indices, (const T*)gates, (T*)out, T_, H, E, K)
+#define FMOE_LAUNCH_EXPERT(N)                                     \
+    do {                                                          \
+        if (act == kActSilu) FMOE_LAUNCH_EXPERT_ACT(N, kActSilu); \
+        else if (act == kActGelu) FMOE_LAUNCH_EXPERT_ACT(N, kActGelu); \
+        else FMOE_LAUNCH_EXPERT_ACT(N, kActNone);                 \
+    } while (0)
     if (nch <= 1) FMOE_LAUNCH_EXPERT(1);
     else if (nch <= 2) FMOE_LAUNCH_EXPERT(2);
     else if (nch <= 4) FMOE_LAUNCH_EXPERT(4);
@@ -123,6 +140,7 @@ int launch_expert_rows(const void* x, const void* down, const void* up, const in
         return FMOE_ERR_UNSUPPORTED;
     }
 #undef FMOE_LAUNCH_EXPERT
+#undef FMOE_LAUNCH_EXPERT_ACT
     FMOE_CHECK_LAUNCH("fmoe_expert_forward");
     return FMOE_OK;
 }
@@ -239,7 +257,7 @@ __global__ __launch_bounds__(256) void expert_scores_slice_kernel(
     }
 }
 
-template <typename T>
+template <typename T, int ACT>
 __global__ __launch_bounds__(256) void expert_gate_kernel(const float* __restrict__ spart, const T* __restrict__ gates,
                                                           const uint32_t* __restrict__ off32, float* __restrict__ a,
                                                           int64_t pairs, int num_slices) {
@@ -247,7 +265,7 @@ __global__ __launch_bounds__(256) void expert_gate_kernel(const float* __restric
     if (p >= pairs) return;
     float s = 0.0f;
     for (int sl = 0; sl < num_slices; ++sl) s += spart[(int64_t)sl * pairs + p];
-    a[p] = off32[p] != kBadOffset ? silu_f32(s) * Elem<T>::to_f32(gates[p]) : 0.0f;
+    a[p] = off32[p] != kBadOffset ? activate<ACT>(s) * Elem<T>::to_f32(gates[p]) : 0.0f;
 }
 
 // acc[0..kVec) += a0 * w0 + a1 * w1 for two 16-byte packets of two different rows
@@ -343,8 +361,8 @@ SlicePlan plan_slices(int64_t T_, int H, int K, size_t elt) {
 
 // Scores, gate and states launches on row offsets that already sit at the start of the workspace.
 template <typename T>
-int launch_expert_slices_prepared(const void* x, const void* down, const void* up, const void* gates, int64_t T_, int H,
-                                  int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+int launch_expert_slices_prepared(int act, const void* x, const void* down, const void* up, const void* gates, int64_t T_,
+                                  int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
     const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
     char* ws = (char*)workspace;
     const uint32_t* off32 = (const uint32_t*)(ws + p.off_idx32);
@@ -353,11 +371,21 @@ int launch_expert_slices_prepared(const void* x, const void* down, const void* u
     float* spart = (float*)(ws + p.off_spart);
     const int64_t pairs = T_ * K;
     const unsigned flat_grid = (unsigned)((pairs + 255) / 256);
-    hipLaunchKernelGGL((expert_scores_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const T*)x, (const T*)down,
-                       table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
-    FMOE_CHECK_LAUNCH("fmoe_expert_forward(scores)");
-    hipLaunchKernelGGL((expert_gate_kernel<T>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
-                       (const T*)gates, off32, a, pairs, p.num_slices);
+    if (act != kActNone) {
+        hipLaunchKernelGGL((expert_scores_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const T*)x, (const T*)down,
+                           table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+        FMOE_CHECK_LAUNCH("fmoe_expert_forward(scores)");
+    }
+    // without a score (product-key memory) the coefficient is the routing weight: no partial sums are read
+    if (act == kActSilu)
+        hipLaunchKernelGGL((expert_gate_kernel<T, kActSilu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
+                           (const T*)gates, off32, a, pairs, p.num_slices);
+    else if (act == kActGelu)
+        hipLaunchKernelGGL((expert_gate_kernel<T, kActGelu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
+                           (const T*)gates, off32, a, pairs, p.num_slices);
+    else
+        hipLaunchKernelGGL((expert_gate_kernel<T, kActNone>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
+                           (const T*)gates, off32, a, pairs, 0);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(gate)");
     hipLaunchKernelGGL((expert_states_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
                        (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
@@ -367,7 +395,7 @@ int launch_expert_slices_prepared(const void* x, const void* down, const void* u
 }
 
 template <typename T>
-int launch_expert_slices(const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
+int launch_expert_slices(int act, const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
                          int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
     const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
     uint32_t* off32 = (uint32_t*)((char*)workspace + p.off_idx32);
@@ -375,7 +403,7 @@ int launch_expert_slices(const void* x, const void* down, const void* up, const 
     hipLaunchKernelGGL(expert_prepare_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, indices, off32,
                        pairs, E, (uint32_t)(H * sizeof(T)));
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(prepare)");
-    return launch_expert_slices_prepared<T>(x, down, up, gates, T_, H, E, K, out, workspace, stream);
+    return launch_expert_slices_prepared<T>(act, x, down, up, gates, T_, H, E, K, out, workspace, stream);
 }
 
 // A 128-byte slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic;
@@ -397,69 +425,101 @@ int expert_slices_prepared(const void* x, const void* down, const void* up, cons
                            int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
                            hipStream_t stream) {
     switch (dtype) {
-        case FMOE_F32: return launch_expert_slices_prepared<float>(x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
-        case FMOE_BF16: return launch_expert_slices_prepared<bf16_t>(x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
-        default: return launch_expert_slices_prepared<f16_t>(x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+        case FMOE_F32: return launch_expert_slices_prepared<float>(kActSilu, x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+        case FMOE_BF16: return launch_expert_slices_prepared<bf16_t>(kActSilu, x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+        default: return launch_expert_slices_prepared<f16_t>(kActSilu, x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
     }
 }
 
 }  // namespace fmoe
 
-extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
+extern "C" size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype,
+                                                   int algo) {
     using namespace fmoe;
-    (void)num_experts;
-    if (num_tokens <= 0 || hidden <= 0 || top_k <= 0 || !dtype_ok(dtype)) return 0;
-    // sized for the column-slice path whichever path a call ends up taking
-    return plan_slices(num_tokens, hidden, top_k, dtype_size(dtype)).bytes;
+    if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0 || top_k <= 0 || !dtype_ok(dtype)) return 0;
+    const bool possible = slices_possible(num_experts, hidden, dtype_size(dtype));
+    const bool slices = algo == FMOE_EXPERT_SLICES || (algo == FMOE_EXPERT_AUTO && possible && slices_pay(num_tokens, num_experts, top_k));
+    return slices ? plan_slices(num_tokens, hidden, top_k, dtype_size(dtype)).bytes : 0;   // the row schedule needs no scratch
 }
 
-extern "C" int fmoe_expert_forward_algo(const void* x, const void* down, const void* up, const int64_t* indices,
-                                        const void* gates, int64_t num_tokens, int hidden, int64_t num_experts,
-                                        int top_k, int dtype, void* out, void* workspace, size_t workspace_bytes,
-                                        int algo, void* stream) {
-    using namespace fmoe;
+extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
+    return fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, dtype, FMOE_EXPERT_AUTO);
+}
+
+namespace fmoe {
+namespace {
+
+// Shared body of the three gather ops; `who` names the entry point in messages, `down` is unused for kActNone.
+int expert_dispatch(const char* who, int act, const void* x, const void* down, const void* up, const int64_t* indices,
+                    const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, void* out,
+                    void* workspace, size_t workspace_bytes, int algo, void* stream) {
     clear_error();
-    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_expert_forward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "%s: unknown dtype %d", who, dtype);
     FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_experts > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
-                 "fmoe_expert_forward: bad shape T=%lld H=%d E=%lld K=%d", (long long)num_tokens, hidden,
+                 "%s: bad shape T=%lld H=%d E=%lld K=%d", who, (long long)num_tokens, hidden,
                  (long long)num_experts, top_k);
     FMOE_REQUIRE(algo >= FMOE_EXPERT_AUTO && algo <= FMOE_EXPERT_SLICES, FMOE_ERR_UNSUPPORTED,
-                 "fmoe_expert_forward: unknown algo %d", algo);
+                 "%s: unknown algo %d", who, algo);
     if (num_tokens == 0) return FMOE_OK;
-    FMOE_REQUIRE(x && down && up && out, FMOE_ERR_NULL_POINTER, "fmoe_expert_forward: null tensor pointer");
+    FMOE_REQUIRE((x || act == kActNone) && (down || act == kActNone) && up && out, FMOE_ERR_NULL_POINTER, "%s: null tensor pointer", who);
     FMOE_REQUIRE(top_k == 0 || (indices && gates), FMOE_ERR_NULL_POINTER,
-                 "fmoe_expert_forward: null indices/gates with top_k=%d", top_k);
+                 "%s: null indices/gates with top_k=%d", who, top_k);
     const int vec = (int)(16 / dtype_size(dtype));
     FMOE_REQUIRE(hidden % vec == 0, FMOE_ERR_ALIGNMENT,
-                 "fmoe_expert_forward: hidden=%d must be a multiple of %d (16-byte rows)", hidden, vec);
+                 "%s: hidden=%d must be a multiple of %d (16-byte rows)", who, hidden, vec);
     FMOE_REQUIRE(aligned16(x) && aligned16(down) && aligned16(up) && aligned16(out), FMOE_ERR_ALIGNMENT,
-                 "fmoe_expert_forward: tensor pointers must be 16-byte aligned");
+                 "%s: tensor pointers must be 16-byte aligned", who);
     FMOE_REQUIRE(num_experts < (1ll << 31) && (int64_t)num_tokens * top_k < (1ll << 40), FMOE_ERR_UNSUPPORTED,
-                 "fmoe_expert_forward: problem too large (E=%lld, pairs=%lld)", (long long)num_experts,
+                 "%s: problem too large (E=%lld, pairs=%lld)", who, (long long)num_experts,
                  (long long)(num_tokens * top_k));
     hipStream_t s = (hipStream_t)stream;
     bool slices = algo == FMOE_EXPERT_SLICES || (algo == FMOE_EXPERT_AUTO && slices_pay(num_tokens, num_experts, top_k));
     if (top_k == 0) slices = false;
     if (slices && !slices_possible(num_experts, hidden, dtype_size(dtype))) {
         FMOE_REQUIRE(algo == FMOE_EXPERT_AUTO, FMOE_ERR_UNSUPPORTED,
-                     "fmoe_expert_forward: tables of 4 GiB or more cannot use the column-slice schedule");
+                     "%s: tables of 4 GiB or more cannot use the column-slice schedule", who);
         slices = false;
     }
     if (slices) {
-        const size_t need = fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, dtype);
+        const size_t need = fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, dtype, FMOE_EXPERT_SLICES);
         FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
-                     "fmoe_expert_forward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+                     "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
         switch (dtype) {
-            case FMOE_F32: return launch_expert_slices<float>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
-            case FMOE_BF16: return launch_expert_slices<bf16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
-            default: return launch_expert_slices<f16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            case FMOE_F32: return launch_expert_slices<float>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            case FMOE_BF16: return launch_expert_slices<bf16_t>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            default: return launch_expert_slices<f16_t>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
         }
     }
     switch (dtype) {
-        case FMOE_F32: return launch_expert_rows<float>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
-        case FMOE_BF16: return launch_expert_rows<bf16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
-        default: return launch_expert_rows<f16_t>(x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+        case FMOE_F32: return launch_expert_rows<float>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+        case FMOE_BF16: return launch_expert_rows<bf16_t>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
+        default: return launch_expert_rows<f16_t>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, s);
     }
+}
+
+}  // namespace
+}  // namespace fmoe
+
+extern "C" int fmoe_expert_forward_algo(const void* x, const void* down, const void* up, const int64_t* indices,
+                                        const void* gates, int64_t num_tokens, int hidden, int64_t num_experts,
+                                        int top_k, int dtype, void* out, void* workspace, size_t workspace_bytes,
+                                        int algo, void* stream) {
+    return fmoe::expert_dispatch("fmoe_expert_forward", fmoe::kActSilu, x, down, up, indices, gates, num_tokens, hidden,
+                                 num_experts, top_k, dtype, out, workspace, workspace_bytes, algo, stream);
+}
+
+extern "C" int fmoe_peer_forward(const void* x, const void* down, const void* up, const void* routing_weights,
+                                 const int64_t* indices, int64_t num_tokens, int hidden, int64_t num_experts, int top_k,
+                                 int dtype, void* out, void* workspace, size_t workspace_bytes, void* stream) {
+    return fmoe::expert_dispatch("fmoe_peer_forward", fmoe::kActGelu, x, down, up, indices, routing_weights, num_tokens, hidden,
+                                 num_experts, top_k, dtype, out, workspace, workspace_bytes, FMOE_EXPERT_AUTO, stream);
+}
+
+extern "C" int fmoe_pkm_forward(const void* values, const void* routing_weights, const int64_t* indices, int64_t num_tokens,
+                                int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    return fmoe::expert_dispatch("fmoe_pkm_forward", fmoe::kActNone, values, values, values, indices, routing_weights, num_tokens,
+                                 hidden, num_experts, top_k, dtype, out, workspace, workspace_bytes, FMOE_EXPERT_AUTO, stream);
 }
 
 extern "C" int fmoe_expert_forward(const void* x, const void* down, const void* up, const int64_t* indices,

@@ -34,6 +34,7 @@ SIGNATURES = {
     "fmoe_router_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int,
                                    _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_expert_workspace_bytes": (_sz, [_i64, _int, _i64, _int, _int]),
+    "fmoe_expert_workspace_bytes_algo": (_sz, [_i64, _int, _i64, _int, _int, _int]),
     "fmoe_expert_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_expert_forward_algo": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _int, _vp]),
     "fmoe_mlp_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
@@ -43,6 +44,8 @@ SIGNATURES = {
                                   _int, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_mlp_gate_up": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
     "fmoe_mlp_down": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp]),
+    "fmoe_peer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
+    "fmoe_pkm_forward": (_int, [_vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_router_topk_backward": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
     "fmoe_swiglu_backward": (_int, [_vp, _vp, _vp, _i64, _int, _int, _vp, _vp, _vp]),
     "fmoe_mlp_backward_workspace_bytes": (_sz, [_i64, _int, _int, _int]),

@@ -36,7 +36,7 @@ def expert_forward(hidden_states, down_weights, up_weights, indices, routing_wei
     code = _C.dtype_code(dtype)
     out = torch.empty_like(x)
     L = _C.lib()
-    ws_bytes = L.fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, code)
+    ws_bytes = L.fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, code, algo)
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8) if ws_bytes else None
     with torch.cuda.device(dev):
         status = L.fmoe_expert_forward_algo(

@@ -106,10 +106,12 @@ int fmoe_router_forward(const void* x, const void* gate_w, void* running_mean, v
  * Duplicate ids in a row add, as in the reference.  An id outside [0,E) contributes nothing (the
  * reference reads out of bounds).  Accumulation is fp32 and deterministic (no atomics); `out` is
  * written once, it need not be zeroed.
- * fmoe_expert_workspace_bytes() gives the scratch the call needs (may be 0); pass a 256-byte aligned
- * buffer of at least that size.
+ * fmoe_expert_workspace_bytes() gives the scratch fmoe_expert_forward needs for these extents (0 when it takes the
+ * row schedule); pass a 256-byte aligned buffer of at least that size.  fmoe_expert_workspace_bytes_algo() gives it
+ * for a schedule forced through fmoe_expert_forward_algo().
  */
 size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
+size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, int algo);
 
 int fmoe_expert_forward(const void* x, const void* down, const void* up, const int64_t* indices,
                         const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k,
@@ -179,6 +181,25 @@ int fmoe_block_forward(const void* x, const void* gate_proj_w, const void* up_pr
                        float eps, int64_t num_tokens, int hidden, int intermediate, int64_t num_experts, int num_keys,
                        int top_k, int dtype, int norm_topk_prob, void* out, void* router_logits, int64_t* indices_out,
                        void* gates_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * The two other gather ops of the reference that share the routed-expert kernels (forward only there too).
+ *
+ * PEER, triton_peer_func / peer_forward (flash_moe/ops/triton/peer.py:246-255, 151-219; eager form tests/test_peer.py:9-24):
+ *   out[t] = sum_k gelu(<x[t], down[idx[t,k]]>) * w[t,k] * up[idx[t,k]]     (erf GELU)
+ * i.e. fmoe_expert_forward with GELU in place of SiLU; note the reference's argument order (weights before indices).
+ *
+ * PKM, triton_pkm_func / pkm_forward (flash_moe/ops/triton/pkm.py:195-200, 123-174; eager form tests/test_pkm.py:9-20):
+ *   out[t] = sum_k w[t,k] * values[idx[t,k]]
+ * Both take a workspace of fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, dtype) bytes.
+ */
+int fmoe_peer_forward(const void* x, const void* down, const void* up, const void* routing_weights, const int64_t* indices,
+                      int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+int fmoe_pkm_forward(const void* values, const void* routing_weights, const int64_t* indices, int64_t num_tokens, int hidden,
+                     int64_t num_experts, int top_k, int dtype, void* out, void* workspace, size_t workspace_bytes,
+                     void* stream);
 
 /* ================================================================================================
  * Backward passes.  Deterministic: no global atomics, every gradient element is written once.

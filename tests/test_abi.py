@@ -95,6 +95,14 @@ def test_expert_argument_checks():
     assert f(a, a, a, a, a, 4, 1 << 20, 16, 2, _C.BF16, a, None, 0, None) == -5      # hidden too large
     assert f(None, None, None, None, None, 0, 64, 16, 2, _C.BF16, None, None, 0, None) == 0
     assert isinstance(lib.fmoe_expert_workspace_bytes(1024, 1024, 16384, 64, _C.BF16), int)
+    # the size follows the schedule: column slices when a slice of the table fits L2 and there are enough pairs, else none
+    sliced = lib.fmoe_expert_workspace_bytes(4096, 1024, 16384, 64, _C.BF16)
+    assert sliced >= 4096 * 64 * (4 + 4 + 16 * 4) and sliced % 256 == 0
+    assert lib.fmoe_expert_workspace_bytes(32768, 2048, 262144, 128, _C.BF16) == 0      # table slice too large for L2
+    assert lib.fmoe_expert_workspace_bytes(64, 1024, 16384, 8, _C.BF16) == 0            # too few pairs
+    assert lib.fmoe_expert_workspace_bytes_algo(64, 1024, 16384, 8, _C.BF16, _C.EXPERT_SLICES) > 0
+    assert lib.fmoe_expert_workspace_bytes_algo(4096, 1024, 16384, 64, _C.BF16, _C.EXPERT_ROWS) == 0
+    assert lib.fmoe_expert_workspace_bytes_algo(4096, 1024, 16384, 64, _C.BF16, _C.EXPERT_AUTO) == sliced
 
 
 def test_mlp_argument_checks():

@@ -178,3 +178,48 @@ def test_mlp_backward_throughput(case):
 
     harness.run([harness.Impl(harness.BASELINE, step(orc.mlp_forward)), harness.Impl(harness.HIP, step(flash_mlp_func))],
                 lambda: args, flops=3 * 6.0 * T * H * I, what=f"mlp forward+backward T={T} H={H} I={I}", repeat=10, validate=validate)
+
+
+PEER_CASES = [(1024, 1024, 102400, 1250), (1024, 1024, 102400, 2500), (1024, 1024, 102400, 6250), (1024, 1024, 102400, 12500),
+              (2048, 1024, 102400, 1250), (4096, 1024, 102400, 1250), (8192, 1024, 102400, 1250), (16384, 1024, 102400, 1250)]
+PKM_CASES = [(1024, 1024, 197136, 2500), (1024, 1024, 197136, 5000), (1024, 1024, 197136, 12500), (1024, 1024, 197136, 25000),
+             (2048, 1024, 197136, 2500), (4096, 1024, 197136, 2500), (8192, 1024, 197136, 2500), (16384, 1024, 197136, 2500)]
+
+
+def chunked(fn, chunk, token_args):
+    """Eager baseline over token chunks (its [chunk, K, H] gathers would not fit otherwise); `token_args` are the
+    positions of the per-token arguments."""
+    def run(*a):
+        T = a[token_args[0]].shape[0]
+        return torch.cat([fn(*[t[lo:lo + chunk] if i in token_args else t for i, t in enumerate(a)]) for lo in range(0, T, chunk)])
+    return run
+
+
+@pytest.mark.parametrize("case", pick(PEER_CASES))
+def test_peer_forward_throughput(case):
+    """Case list of the reference's tests/test_peer.py:226-237."""
+    from flash_moe.ops.triton.peer import triton_peer_func
+    from test_peer_pkm_gpu import peer_reference
+
+    T, H, E, K = case
+    x, wd, wu, idx, w = expert_inputs(T, H, E, K, torch.bfloat16)
+    chunk = max(1, (1 << 28) // (K * H))
+    with torch.no_grad():
+        harness.run([harness.Impl(harness.BASELINE, chunked(peer_reference, chunk, (0, 3, 4))),
+                     harness.Impl(harness.HIP, triton_peer_func)], lambda: (x, wd, wu, w, idx),
+                    flops=4.0 * T * H * K, what=f"peer forward T={T} H={H} E={E} K={K}", repeat=5)
+
+
+@pytest.mark.parametrize("case", pick(PKM_CASES))
+def test_pkm_forward_throughput(case):
+    """Case list of the reference's tests/test_pkm.py:170-181."""
+    from flash_moe.ops.triton.pkm import triton_pkm_func
+    from test_peer_pkm_gpu import pkm_reference
+
+    T, H, E, K = case
+    _, values, _, idx, w = expert_inputs(T, H, E, K, torch.bfloat16)
+    chunk = max(1, (1 << 28) // (K * H))
+    with torch.no_grad():
+        harness.run([harness.Impl(harness.BASELINE, chunked(pkm_reference, chunk, (1, 2))),
+                     harness.Impl(harness.HIP, triton_pkm_func)], lambda: (values, w, idx),
+                    flops=2.0 * T * H * K, what=f"pkm forward T={T} H={H} E={E} K={K}", repeat=5)
