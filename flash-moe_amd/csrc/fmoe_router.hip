@@ -38,26 +38,19 @@ __device__ inline uint64_t make_key(float score, uint32_t index) {
 __device__ inline float key_score(uint64_t k) { return order_value((uint32_t)(k >> 32)); }
 __device__ inline uint32_t key_index(uint64_t k) { return ~(uint32_t)(k & 0xffffffffu); }
 
-// Value of lane (lane ^ mask) for mask in {1,2,4,8,16,32}, without going through LDS: DPP inside a row of 16 lanes,
-// v_permlane16_swap / v_permlane32_swap across rows.  `mask` must be a compile-time constant after inlining.
+// Value of lane (lane ^ mask) for mask in {1,2,4,8,16,32}; `mask` must be a compile-time constant after inlining.
+// Distances 1, 2 and 8 are single DPP moves.  Distances 4, 16 and 32 would cost 2-4 vector instructions each on the
+// DPP / permlane path; the kernel is bound by vector-ALU issue, so they go through the LDS crossbar instead
+// (ds_swizzle / ds_bpermute: no LDS memory is touched, no vector-ALU slot is used, other waves cover the latency).
 __device__ inline uint32_t xor_lane_u32(uint32_t v, int mask, int lane) {
     const int iv = (int)v;
     switch (mask) {
         case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, iv, 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
         case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, iv, 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
-        case 4: {
-            int t = __builtin_amdgcn_update_dpp(0, iv, 0x104, 0xF, 0x5, false);               // row_shl:4 into banks 0,2
-            return (uint32_t)__builtin_amdgcn_update_dpp(t, iv, 0x114, 0xF, 0xA, false);      // row_shr:4 into banks 1,3
-        }
+        case 4: return (uint32_t)__builtin_amdgcn_ds_swizzle(iv, (4 << 10) | 0x1F);          // bit mode: lane ^ 4
         case 8: return (uint32_t)__builtin_amdgcn_update_dpp(0, iv, 0x128, 0xF, 0xF, true);   // row_ror:8
-        case 16: {
-            const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);   // odd rows of [0] <-> even rows of [1]
-            return (lane & 16) ? r[0] : r[1];
-        }
-        default: {
-            const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);   // upper half of [0] <-> lower half of [1]
-            return (lane & 32) ? r[0] : r[1];
-        }
+        case 16: return (uint32_t)__builtin_amdgcn_ds_swizzle(iv, (16 << 10) | 0x1F);        // bit mode: lane ^ 16
+        default: return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, iv);
     }
 }
 __device__ inline uint64_t xor_lane_u64(uint64_t v, int mask, int lane) {
