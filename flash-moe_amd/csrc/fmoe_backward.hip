@@ -526,7 +526,8 @@ extern "C" int fmoe_expert_backward(const void* dout, const void* x, const void*
                  hidden, 8 * kWave * vec);
     FMOE_REQUIRE(num_experts < (1ll << 31) - 1 && (int64_t)num_tokens * top_k < (1ll << 31), FMOE_ERR_UNSUPPORTED,
                  "fmoe_expert_backward: E=%lld or T*K=%lld >= 2^31", (long long)num_experts, (long long)num_tokens * top_k);
-    FMOE_REQUIRE(dx && ddown && dup && x && dout && down && up, FMOE_ERR_NULL_POINTER, "fmoe_expert_backward: null tensor pointer");
+    FMOE_REQUIRE(ddown && dup && down && up && (num_tokens == 0 || (dx && x && dout)), FMOE_ERR_NULL_POINTER,
+                 "fmoe_expert_backward: null tensor pointer");
     FMOE_REQUIRE(aligned16(dx) && aligned16(ddown) && aligned16(dup) && aligned16(x) && aligned16(dout) && aligned16(down) && aligned16(up),
                  FMOE_ERR_ALIGNMENT, "fmoe_expert_backward: tensor pointers must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;

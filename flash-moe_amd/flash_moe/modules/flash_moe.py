@@ -91,19 +91,19 @@ class FlashMoE(nn.Module):
         if torch.is_grad_enabled() and (hidden_states.requires_grad or any(p.requires_grad for p in self.parameters())):
             return self.forward_autograd(hidden_states)
         bsz, seq_len, _ = hidden_states.shape
-        tokens = hidden_states.reshape(-1, self.hidden_size)
+        tokens = hidden_states.reshape(bsz * seq_len, self.hidden_size)
         out, logits = block_forward(
             tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, self.router_gate.weight,
             self.router_norm, self.down_embed.weight, self.up_embed.weight, self.num_keys, self.top_k, self.norm_topk_prob,
         )
         router_logits = logits.view(tokens.shape[0], 2, self.num_keys).transpose(0, 1)
-        return out.view(bsz, seq_len, -1), router_logits
+        return out.view(bsz, seq_len, self.hidden_size), router_logits
 
     def forward_autograd(self, hidden_states: torch.Tensor):
         """Differentiable forward.  Routing is evaluated in fp32 as on the fused path: the normalised activations are
         rounded to the module dtype, their product with the router gate and the log-softmax are fp32."""
         bsz, seq_len, _ = hidden_states.shape
-        tokens = hidden_states.reshape(-1, self.hidden_size)
+        tokens = hidden_states.reshape(bsz * seq_len, self.hidden_size)
         num_tokens = tokens.shape[0]
         query = self.router_norm(tokens)
         logits32 = F.linear(query.float(), self.router_gate.weight.float())
@@ -115,15 +115,15 @@ class FlashMoE(nn.Module):
             gates = gates / gates.sum(dim=-1, keepdim=True)
         experts_states = flash_expert_func(tokens, self.down_embed.weight, self.up_embed.weight, indices, gates.to(tokens.dtype))
         out = flash_mlp_func(tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight) + experts_states
-        return out.view(bsz, seq_len, -1), router_logits
+        return out.view(bsz, seq_len, self.hidden_size), router_logits
 
     def forward_staged(self, hidden_states: torch.Tensor):
         """``forward`` as three library calls (router, experts, MLP) instead of one; same results."""
         bsz, seq_len, _ = hidden_states.shape
-        tokens = hidden_states.reshape(-1, self.hidden_size)
+        tokens = hidden_states.reshape(bsz * seq_len, self.hidden_size)
         router_logits, _, indices, gates = self.route(tokens)
         experts_states = expert_forward(tokens, self.down_embed.weight, self.up_embed.weight, indices, gates)
         out = mlp_forward(
             tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, residual=experts_states
         )
-        return out.view(bsz, seq_len, -1), router_logits
+        return out.view(bsz, seq_len, self.hidden_size), router_logits

@@ -232,3 +232,19 @@ def test_block_backward_c4_full_size_properties():
     used[indices.flatten()] = True
     assert (gp["down_embed.weight"][~used] == 0).all() and (gp["up_embed.weight"][~used] == 0).all()
     assert (gp["up_embed.weight"][used].abs().sum(-1) > 0).all()
+
+
+def test_backward_of_empty_batches():
+    from flash_moe.ops.hip.flash_expert import expert_backward
+    from flash_moe.ops.hip.flash_mlp import mlp_backward
+    from flash_moe.ops.hip.flash_router import router_topk_backward
+
+    H, E, K, I, nk = 64, 32, 4, 128, 8
+    z = lambda *s: torch.zeros(*s, device="cuda")
+    assert router_topk_backward(z(0, K), torch.zeros(0, K, dtype=torch.int64, device="cuda"), nk).shape == (2, 0, nk)
+    wd, wu = torch.randn(E, H, device="cuda"), torch.randn(E, H, device="cuda")
+    dx, dwd, dwu, dg = expert_backward(z(0, H), z(0, H), wd, wu, torch.zeros(0, K, dtype=torch.int64, device="cuda"), z(0, K))
+    assert dx.shape == (0, H) and dg.shape == (0, K) and (dwd == 0).all() and (dwu == 0).all()
+    dx, dwg, dwu2, dwd2 = mlp_backward(z(0, H), z(0, H), torch.randn(I, H, device="cuda"), torch.randn(I, H, device="cuda"),
+                                       torch.randn(H, I, device="cuda"))
+    assert dx.shape == (0, H) and (dwg == 0).all() and (dwu2 == 0).all() and (dwd2 == 0).all()

@@ -220,3 +220,10 @@ def test_block_c5_full_size_sampled_tokens():
     y64 = e64 + orc.mlp_forward(xs.cpu().double(), m.gate_proj.weight.cpu().double(), m.up_proj.weight.cpu().double(),
                                 m.down_proj.weight.cpu().double())
     assert_output_close(y[pick], y64.to(dtype), dtype, "C5 block output vs float64 oracle on sampled tokens")
+
+
+def test_block_of_an_empty_batch():
+    m, _ = build(128, 256, 1024, 8, False, torch.bfloat16)
+    m.eval()
+    y, logits = m(torch.zeros(2, 0, 128, device="cuda", dtype=torch.bfloat16))
+    assert y.shape == (2, 0, 128) and logits.shape == (2, 0, 32)
