@@ -160,6 +160,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
                     if (row < M && col < N) {
                         const float g = acc[i][j][v], u = acc[i][j + NF / 2][v];
                         C[(int64_t)row * N + col] = Elem<T>::from_f32(silu_f32(g) * u);
+                        if (R != nullptr) {   // planes [0] and [1] of a [2, M, N] buffer keep the two products
+                            const_cast<T*>(R)[(int64_t)row * N + col] = Elem<T>::from_f32(g);
+                            const_cast<T*>(R)[((int64_t)M + row) * N + col] = Elem<T>::from_f32(u);
+                        }
                     }
                 }
             }
@@ -376,6 +380,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
             __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, t), c_rsrc, lane_bytes, uni_bytes, 0);
         };
         if (EPI == kEpiSwiGLU) {
+            if (R != nullptr) {
+                // keep the gate and up products for a backward pass: planes [0] and [1] of a [2, M, N] buffer
+                T* planes = const_cast<T*>(R);
+                auto g_rsrc = __builtin_amdgcn_make_buffer_rsrc(planes + wave_off, 0, span32, 0x00020000);
+                auto u_rsrc = __builtin_amdgcn_make_buffer_rsrc(planes + (int64_t)M * N + wave_off, 0, span32, 0x00020000);
+#pragma unroll
+                for (int i = 0; i < MF; ++i)
+#pragma unroll
+                    for (int j = 0; j < NF / 2; ++j)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int uni = ((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T);
+                            const T g = Elem<T>::from_f32(acc[i][j][v]), u = Elem<T>::from_f32(acc[i][j + NF / 2][v]);
+                            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, g), g_rsrc, lane_bytes, uni, 0);
+                            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, u), u_rsrc, lane_bytes, uni, 0);
+                        }
+            }
 #pragma unroll
             for (int i = 0; i < MF; ++i)
 #pragma unroll
@@ -458,6 +479,10 @@ __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__
             if (row < M && col < N) {
                 float r = (EPI == kEpiSwiGLU) ? silu_f32(accg[i][j]) * accu[i][j] : accg[i][j];
                 if (EPI == kEpiPlain && R != nullptr) r += R[(int64_t)row * N + col];
+                if (EPI == kEpiSwiGLU && R != nullptr) {
+                    const_cast<float*>(R)[(int64_t)row * N + col] = accg[i][j];
+                    const_cast<float*>(R)[((int64_t)M + row) * N + col] = accu[i][j];
+                }
                 C[(int64_t)row * N + col] = r;
             }
         }
@@ -496,15 +521,15 @@ void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, 
 }
 
 template <typename T>
-int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, hipStream_t stream) {
-    const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu;
+int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
+    const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu, *S = (const T*)saved;
     const bool k_ok = H % 64 == 0;
     if (k_ok && M % 256 == 0 && I % 128 == 0 && (int64_t)(M / 256) * (I / 128) >= 256)
-        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, nullptr, M, I, H, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, S, M, I, H, stream);
     else if (k_ok && M % 128 == 0 && I % 64 == 0)
-        launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, (int64_t)(M / 128) * (I / 64), stream);
+        launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, (int64_t)(M / 128) * (I / 64), stream);
     else
-        launch_gemm<T, 128, 128, kEpiSwiGLU>(A, G, U, (T*)h, nullptr, M, I, H, stream);
+        launch_gemm<T, 128, 128, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up)");
     return FMOE_OK;
 }
@@ -523,9 +548,9 @@ int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* r
     return FMOE_OK;
 }
 
-int gate_up_f32(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, hipStream_t stream) {
+int gate_up_f32(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
     hipLaunchKernelGGL((sgemm_nt_kernel<kEpiSwiGLU>), dim3((I + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
-                       (const float*)x, (const float*)wg, (const float*)wu, (float*)h, nullptr, M, I, H);
+                       (const float*)x, (const float*)wg, (const float*)wu, (float*)h, (const float*)saved, M, I, H);
     FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up, f32)");
     return FMOE_OK;
 }
@@ -556,22 +581,41 @@ extern "C" size_t fmoe_mlp_workspace_bytes(int64_t num_tokens, int hidden, int i
     return fmoe::round_up((size_t)num_tokens * (size_t)intermediate * fmoe::dtype_size(dtype), 256);
 }
 
-extern "C" int fmoe_mlp_gate_up(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
-                                int intermediate, int dtype, void* act, void* stream) {
-    using namespace fmoe;
+namespace fmoe {
+namespace {
+int mlp_gate_up_impl(const char* who, const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
+                     int intermediate, int dtype, void* act, void* saved, void* stream) {
     clear_error();
-    if (int rc = check_mlp_shape("fmoe_mlp_gate_up", num_tokens, hidden, intermediate, dtype)) return rc;
+    if (int rc = check_mlp_shape(who, num_tokens, hidden, intermediate, dtype)) return rc;
     if (num_tokens == 0) return FMOE_OK;
-    FMOE_REQUIRE(x && gate_w && up_w && act, FMOE_ERR_NULL_POINTER, "fmoe_mlp_gate_up: null tensor pointer");
-    FMOE_REQUIRE(dtype == FMOE_F32 || (aligned16(x) && aligned16(gate_w) && aligned16(up_w) && aligned16(act)),
-                 FMOE_ERR_ALIGNMENT, "fmoe_mlp_gate_up: tensor pointers must be 16-byte aligned");
+    FMOE_REQUIRE(x && gate_w && up_w && act, FMOE_ERR_NULL_POINTER, "%s: null tensor pointer", who);
+    FMOE_REQUIRE(dtype == FMOE_F32 || (aligned16(x) && aligned16(gate_w) && aligned16(up_w) && aligned16(act) && aligned16(saved)),
+                 FMOE_ERR_ALIGNMENT, "%s: tensor pointers must be 16-byte aligned", who);
     hipStream_t s = (hipStream_t)stream;
     const int M = (int)num_tokens;
     switch (dtype) {
-        case FMOE_F32: return gate_up_f32(x, gate_w, up_w, M, hidden, intermediate, act, s);
-        case FMOE_BF16: return gate_up_16bit<bf16_t>(x, gate_w, up_w, M, hidden, intermediate, act, s);
-        default: return gate_up_16bit<f16_t>(x, gate_w, up_w, M, hidden, intermediate, act, s);
+        case FMOE_F32: return gate_up_f32(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
+        case FMOE_BF16: return gate_up_16bit<bf16_t>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
+        default: return gate_up_16bit<f16_t>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
     }
+}
+}  // namespace
+}  // namespace fmoe
+
+extern "C" int fmoe_mlp_gate_up(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
+                                int intermediate, int dtype, void* act, void* stream) {
+    return fmoe::mlp_gate_up_impl("fmoe_mlp_gate_up", x, gate_w, up_w, num_tokens, hidden, intermediate, dtype, act, nullptr, stream);
+}
+
+extern "C" int fmoe_mlp_gate_up_save(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
+                                     int intermediate, int dtype, void* act, void* saved, void* stream) {
+    using namespace fmoe;
+    if (saved == nullptr && num_tokens > 0) {
+        clear_error();
+        set_error("fmoe_mlp_gate_up_save: null buffer for the gate and up products");
+        return FMOE_ERR_NULL_POINTER;
+    }
+    return mlp_gate_up_impl("fmoe_mlp_gate_up_save", x, gate_w, up_w, num_tokens, hidden, intermediate, dtype, act, saved, stream);
 }
 
 extern "C" int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int hidden, int intermediate,

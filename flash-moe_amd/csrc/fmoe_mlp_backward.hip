@@ -1,7 +1,7 @@
 // Backward of the shared SwiGLU MLP  y = (silu(x Wg^T) * (x Wu^T)) Wd^T  for gfx950.
 //
-// The forward keeps only silu(a) * b; the gate and up products a, b are recomputed here (two launches of the
-// forward's own NT GEMM), as the reference recomputes the SiLU in its backward.  The SwiGLU gradient is the fused
+// The forward keeps only silu(a) * b unless it was asked to keep the gate and up products a, b as well
+// (fmoe_mlp_gate_up_save); without them they are recomputed here (two launches of the forward's own NT GEMM).  The SwiGLU gradient is the fused
 // elementwise kernel of fmoe_backward.hip (it also rebuilds h = silu(a) * b for dWd).  The remaining products are
 // plain GEMMs in layouts the forward never needs (A B and A^T B); they go to rocBLAS, which is loaded on first use so
 // that the forward path carries no dependency on it:
@@ -108,7 +108,7 @@ extern "C" size_t fmoe_mlp_backward_workspace_bytes(int64_t num_tokens, int hidd
 }
 
 extern "C" int fmoe_mlp_backward(const void* dy, const void* x, const void* gate_w, const void* up_w, const void* down_w,
-                                 int64_t num_tokens, int hidden, int intermediate, int dtype, void* dx, void* dgate_w, void* dup_w,
+                                 const void* saved_products, int64_t num_tokens, int hidden, int intermediate, int dtype, void* dx, void* dgate_w, void* dup_w,
                                  void* ddown_w, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace fmoe;
     clear_error();
@@ -131,11 +131,18 @@ extern "C" int fmoe_mlp_backward(const void* dy, const void* x, const void* gate
     const int T_ = (int)num_tokens, H = hidden, I = intermediate;
     const size_t elt = dtype_size(dtype);
 
-    // a = x Wg^T, b = x Wu^T with the forward's NT kernel ("down" form: out[T,N] = act[T,K] W[N,K]^T)
-    int rc = fmoe_mlp_down(x, gate_w, num_tokens, I, H, dtype, nullptr, a, stream);
-    if (rc) return rc;
-    rc = fmoe_mlp_down(x, up_w, num_tokens, I, H, dtype, nullptr, b, stream);
-    if (rc) return rc;
+    int rc = FMOE_OK;
+    if (saved_products != nullptr) {
+        // the forward kept a = x Wg^T and b = x Wu^T (fmoe_mlp_gate_up_save): planes [0] and [1] of a [2, T, I] buffer
+        a = const_cast<void*>(saved_products);
+        b = (char*)a + (size_t)num_tokens * I * elt;
+    } else {
+        // recompute them with the forward's NT kernel ("down" form: out[T,N] = act[T,K] W[N,K]^T)
+        rc = fmoe_mlp_down(x, gate_w, num_tokens, I, H, dtype, nullptr, a, stream);
+        if (rc) return rc;
+        rc = fmoe_mlp_down(x, up_w, num_tokens, I, H, dtype, nullptr, b, stream);
+        if (rc) return rc;
+    }
 
     std::lock_guard<std::mutex> guard(api().lock);
     rocblas_handle handle = nullptr;

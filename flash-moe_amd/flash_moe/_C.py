@@ -43,13 +43,14 @@ SIGNATURES = {
     "fmoe_block_forward": (_int, [_vp] * 10 + [_int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int, _i64, _int, _int,
                                   _int, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_mlp_gate_up": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
+    "fmoe_mlp_gate_up_save": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp]),
     "fmoe_mlp_down": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp]),
     "fmoe_peer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_pkm_forward": (_int, [_vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_router_topk_backward": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
     "fmoe_swiglu_backward": (_int, [_vp, _vp, _vp, _i64, _int, _int, _vp, _vp, _vp]),
     "fmoe_mlp_backward_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
-    "fmoe_mlp_backward": (_int, [_vp] * 5 + [_i64, _int, _int, _int] + [_vp] * 5 + [_sz, _vp]),
+    "fmoe_mlp_backward": (_int, [_vp] * 6 + [_i64, _int, _int, _int] + [_vp] * 5 + [_sz, _vp]),
     "fmoe_expert_backward_workspace_bytes": (_sz, [_i64, _int, _i64, _int, _int]),
     "fmoe_expert_backward": (_int, [_vp] * 6 + [_i64, _int, _i64, _int, _int] + [_vp] * 5 + [_sz, _vp]),
 }

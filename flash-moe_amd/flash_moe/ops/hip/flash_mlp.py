@@ -48,10 +48,35 @@ def mlp_forward(x, gate_weight, up_weight, down_weight, residual: Optional[torch
     return out.view(x.shape)
 
 
-def mlp_backward(dout, x, gate_weight, up_weight, down_weight):
+def mlp_forward_saving(x, gate_weight, up_weight, down_weight):
+    """``mlp_forward`` that also returns the [2, T, I] gate and up products for ``mlp_backward`` (``fmoe_mlp_gate_up_save``
+    then ``fmoe_mlp_down``), as the reference's SwiGLU function saves them (flash_moe/ops/triton/flash_mlp.py:153-159)."""
+    hidden, inter = x.shape[-1], gate_weight.shape[0]
+    if gate_weight.shape != (inter, hidden) or up_weight.shape != (inter, hidden) or down_weight.shape != (hidden, inter):
+        raise ValueError("expected gate_weight/up_weight (intermediate, hidden) and down_weight (hidden, intermediate)")
+    if any(t.dtype != x.dtype for t in (gate_weight, up_weight, down_weight)):
+        raise TypeError(f"all weights must have the dtype of x ({x.dtype})")
+    dev = _C.require_gpu(x, gate_weight, up_weight, down_weight)
+    x2 = x.contiguous().view(-1, hidden)
+    wg, wu, wd = gate_weight.contiguous(), up_weight.contiguous(), down_weight.contiguous()
+    num_tokens, code = x2.shape[0], _C.dtype_code(x.dtype)
+    act = torch.empty((num_tokens, inter), device=dev, dtype=x.dtype)
+    saved = torch.empty((2, num_tokens, inter), device=dev, dtype=x.dtype)
+    out = torch.empty_like(x2)
+    L = _C.lib()
+    with torch.cuda.device(dev):
+        stream = _C.current_stream(dev)
+        _C.check(L.fmoe_mlp_gate_up_save(_C.ptr(x2), _C.ptr(wg), _C.ptr(wu), num_tokens, hidden, inter, code, _C.ptr(act),
+                                         _C.ptr(saved), stream), "flash_mlp")
+        _C.check(L.fmoe_mlp_down(_C.ptr(act), _C.ptr(wd), num_tokens, hidden, inter, code, None, _C.ptr(out), stream), "flash_mlp")
+    return out.view(x.shape), saved
+
+
+def mlp_backward(dout, x, gate_weight, up_weight, down_weight, saved=None):
     """Gradients ``(dx, dgate_weight, dup_weight, ddown_weight)`` of ``mlp_forward`` without residual
-    (``fmoe_mlp_backward``): the gate and up products are recomputed, the SwiGLU gradient is the fused kernel behind
-    ``swiglu_backward``, the transposed-operand GEMMs are rocBLAS calls inside the library."""
+    (``fmoe_mlp_backward``): the gate and up products come from ``saved`` (``mlp_forward_saving``) or are recomputed, the
+    SwiGLU gradient is the fused kernel behind ``swiglu_backward``, the transposed-operand GEMMs are rocBLAS calls
+    inside the library."""
     hidden, inter = x.shape[-1], gate_weight.shape[0]
     dev = _C.require_gpu(dout, x, gate_weight, up_weight, down_weight)
     if dout.shape != x.shape or dout.dtype != x.dtype:
@@ -60,6 +85,8 @@ def mlp_backward(dout, x, gate_weight, up_weight, down_weight):
     wg, wu, wd = gate_weight.contiguous(), up_weight.contiguous(), down_weight.contiguous()
     num_tokens = x2.shape[0]
     code = _C.dtype_code(x.dtype)
+    if saved is not None and (saved.shape != (2, num_tokens, inter) or saved.dtype != x.dtype or not saved.is_contiguous()):
+        raise ValueError("saved must be the contiguous [2, T, I] tensor mlp_forward_saving returned")
     dx, dwg, dwu, dwd = torch.empty_like(x2), torch.empty_like(wg), torch.empty_like(wu), torch.empty_like(wd)
     if num_tokens == 0:
         return dx.view(x.shape), dwg.zero_(), dwu.zero_(), dwd.zero_()
@@ -68,7 +95,7 @@ def mlp_backward(dout, x, gate_weight, up_weight, down_weight):
     ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
     with torch.cuda.device(dev):
         status = L.fmoe_mlp_backward(
-            _C.ptr(dy), _C.ptr(x2), _C.ptr(wg), _C.ptr(wu), _C.ptr(wd), num_tokens, hidden, inter, code, _C.ptr(dx),
+            _C.ptr(dy), _C.ptr(x2), _C.ptr(wg), _C.ptr(wu), _C.ptr(wd), _C.ptr(saved), num_tokens, hidden, inter, code, _C.ptr(dx),
             _C.ptr(dwg), _C.ptr(dwu), _C.ptr(dwd), _C.ptr(ws), ws_bytes, _C.current_stream(dev),
         )
     _C.check(status, "flash_mlp backward")
@@ -94,13 +121,17 @@ class FlashMLPFunc(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def forward(ctx, x, gate_weight, up_weight, down_weight):
-        ctx.save_for_backward(x, gate_weight, up_weight, down_weight)
-        return mlp_forward(x, gate_weight, up_weight, down_weight)
+        if not any(ctx.needs_input_grad) or x.numel() == 0:
+            return mlp_forward(x, gate_weight, up_weight, down_weight)
+        out, saved = mlp_forward_saving(x, gate_weight, up_weight, down_weight)
+        ctx.save_for_backward(x, gate_weight, up_weight, down_weight, saved)
+        return out
 
     @staticmethod
     @ensure_contiguous
     def backward(ctx, dout):
-        return mlp_backward(dout, *ctx.saved_tensors)
+        x, gate_weight, up_weight, down_weight, saved = ctx.saved_tensors
+        return mlp_backward(dout, x, gate_weight, up_weight, down_weight, saved)
 
 
 def flash_mlp_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor, down_weight: torch.Tensor) -> torch.Tensor:

@@ -156,6 +156,10 @@ int fmoe_mlp_forward(const void* x, const void* gate_w, const void* up_w, const 
  *   fmoe_mlp_down:    out = act down_w^T [+ residual]          -- its last matmul (flash_mlp.py:173-181) */
 int fmoe_mlp_gate_up(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
                      int intermediate, int dtype, void* act, void* stream);
+/* fmoe_mlp_gate_up that also keeps the two products for a backward pass, as TritonSwiGLUFunc.forward saves a and b
+ * (flash_moe/ops/triton/flash_mlp.py:153-159): saved [2,T,I] dtype, plane 0 = x gate_w^T, plane 1 = x up_w^T. */
+int fmoe_mlp_gate_up_save(const void* x, const void* gate_w, const void* up_w, int64_t num_tokens, int hidden,
+                          int intermediate, int dtype, void* act, void* saved, void* stream);
 
 int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int hidden, int intermediate, int dtype,
                   const void* residual, void* out, void* stream);
@@ -219,12 +223,13 @@ int fmoe_swiglu_backward(const void* dc, const void* a, const void* b, int64_t r
 
 /* Backward of triton_flash_mlp_func (flash_moe/ops/triton/flash_mlp.py:169-181: two matmuls, TritonSwiGLUFunc, one
  * matmul, differentiated by autograd in the reference): from dy [T,H] the gradients dx [T,H], dgate_w, dup_w [I,H],
- * ddown_w [H,I].  The gate and up products are recomputed; the transposed-operand GEMMs are rocBLAS calls (loaded on
- * first use; FMOE_ERR_LIBRARY if unavailable). */
+ * ddown_w [H,I].  saved_products: the [2,T,I] buffer fmoe_mlp_gate_up_save() filled in the forward, or NULL to
+ * recompute the gate and up products here.  The transposed-operand GEMMs are rocBLAS calls (loaded on first use;
+ * FMOE_ERR_LIBRARY if unavailable). */
 size_t fmoe_mlp_backward_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int dtype);
 
 int fmoe_mlp_backward(const void* dy, const void* x, const void* gate_w, const void* up_w, const void* down_w,
-                      int64_t num_tokens, int hidden, int intermediate, int dtype, void* dx, void* dgate_w, void* dup_w,
+                      const void* saved_products, int64_t num_tokens, int hidden, int intermediate, int dtype, void* dx, void* dgate_w, void* dup_w,
                       void* ddown_w, void* workspace, size_t workspace_bytes, void* stream);
 
 /* FlashExpertFunc.backward / _flash_expert_backward (flash_moe/ops/triton/flash_expert.py:654-745, kernels :234-525):

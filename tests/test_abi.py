@@ -181,7 +181,7 @@ def test_backward_argument_checks():
     mb = lib.fmoe_mlp_backward
 
     def mcall(T=8, H=64, I=128, dtype=_C.BF16, dy=a, ws_bytes=mneed):
-        return mb(dy, a, a, a, a, T, H, I, dtype, a, a, a, a, a, ws_bytes, None)
+        return mb(dy, a, a, a, a, None, T, H, I, dtype, a, a, a, a, a, ws_bytes, None)
 
     assert mcall(dtype=5) == -4
     assert mcall(T=0) == -2

@@ -248,3 +248,20 @@ def test_backward_of_empty_batches():
     dx, dwg, dwu2, dwd2 = mlp_backward(z(0, H), z(0, H), torch.randn(I, H, device="cuda"), torch.randn(I, H, device="cuda"),
                                        torch.randn(H, I, device="cuda"))
     assert dx.shape == (0, H) and (dwg == 0).all() and (dwu2 == 0).all() and (dwd2 == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
+    from flash_moe.ops.hip.flash_mlp import mlp_backward, mlp_forward, mlp_forward_saving
+
+    T, H, I = 256, 256, 512
+    x = torch.randn(T, H, generator=gen(1)).to(dtype).cuda()
+    wg, wu, wd = ((torch.randn(s, generator=gen(k)) * 0.05).to(dtype).cuda() for k, s in ((2, (I, H)), (3, (I, H)), (4, (H, I))))
+    dy = torch.randn(T, H, generator=gen(5)).to(dtype).cuda()
+    out, saved = mlp_forward_saving(x, wg, wu, wd)
+    assert torch.equal(out, mlp_forward(x, wg, wu, wd)) and saved.shape == (2, T, I)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    torch.testing.assert_close(saved[0].float(), x.float() @ wg.float().t(), rtol=tol, atol=tol)
+    torch.testing.assert_close(saved[1].float(), x.float() @ wu.float().t(), rtol=tol, atol=tol)
+    for a, b in zip(mlp_backward(dy, x, wg, wu, wd, saved), mlp_backward(dy, x, wg, wu, wd)):
+        assert rel_fro(a, b) < (1e-6 if dtype == torch.float32 else 2e-3)
