@@ -72,28 +72,6 @@ int launch_router_backward(const void* dscores, const int64_t* indices, void* dl
 // ------------------------------------------------------------------------------------------------------------
 // SwiGLU
 // ------------------------------------------------------------------------------------------------------------
-template <typename T> __device__ inline void unpack16(u32x4_t w, float* v);
-template <> __device__ inline void unpack16<float>(u32x4_t w, float* v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(w[i]);
-}
-template <> __device__ inline void unpack16<bf16_t>(u32x4_t w, float* v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        v[2 * i] = __uint_as_float(w[i] << 16);
-        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-    }
-}
-template <> __device__ inline void unpack16<f16_t>(u32x4_t w, float* v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t wi = w[i];
-        const f16x2_t p = __builtin_bit_cast(f16x2_t, wi);
-        v[2 * i] = (float)p[0];
-        v[2 * i + 1] = (float)p[1];
-    }
-}
-
 // One 16-byte packet per thread.  Row strides (elements) let da / db / h live side by side in wider buffers.
 template <typename T>
 __global__ __launch_bounds__(256) void swiglu_backward_kernel(const T* __restrict__ dc, const T* __restrict__ a,

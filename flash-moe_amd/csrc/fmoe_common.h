@@ -57,6 +57,12 @@ int expert_slices_prepared(const void* x, const void* down, const void* up, cons
                            int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
                            hipStream_t stream);
 
+// Plain library GEMM (rocBLAS, loaded on first use) for the operand layouts of the backward passes; row-major
+// C[M,N] = A[M,K] B[K,N] (kBlasNN) or A[K,M]^T B[K,N] (kBlasTN), C = product + beta * C.  Defined in fmoe_mlp_backward.hip.
+enum { kBlasNN = 0, kBlasTN = 1 };
+int blas_gemm(int layout, int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C, int ldc, float beta,
+              int dtype, hipStream_t stream);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline size_t dtype_size(int dtype) { return dtype == FMOE_F32 ? 4 : 2; }
 inline bool dtype_ok(int dtype) { return dtype == FMOE_F32 || dtype == FMOE_BF16 || dtype == FMOE_F16; }

@@ -54,32 +54,19 @@ int rocblas_for_device(rocblas_handle* out) {
         }
     }
     FMOE_REQUIRE(r.create_handle && r.set_stream && r.gemm_ex, FMOE_ERR_LIBRARY,
-                 "fmoe_mlp_backward: rocBLAS (librocblas.so) could not be loaded: %s", dlerror() ? dlerror() : "missing symbols");
+                 "rocBLAS (librocblas.so) could not be loaded: %s", dlerror() ? dlerror() : "missing symbols");
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
-    FMOE_REQUIRE(e == hipSuccess && dev >= 0 && dev < 64, FMOE_ERR_LIBRARY, "fmoe_mlp_backward: no current device");
+    FMOE_REQUIRE(e == hipSuccess && dev >= 0 && dev < 64, FMOE_ERR_LIBRARY, "no current HIP device for rocBLAS");
     if (!r.handle[dev]) {
         const rocblas_status st = r.create_handle(&r.handle[dev]);
-        FMOE_REQUIRE(st == rocblas_status_success, FMOE_ERR_LIBRARY, "fmoe_mlp_backward: rocblas_create_handle failed (%d)", (int)st);
+        FMOE_REQUIRE(st == rocblas_status_success, FMOE_ERR_LIBRARY, "rocblas_create_handle failed (%d)", (int)st);
     }
     *out = r.handle[dev];
     return FMOE_OK;
 }
 
-enum Layout { kNN, kTN };   // row-major C[M,N] = A[M,K] B[K,N]   |   C[M,N] = A[K,M]^T B[K,N]
-
-// Row-major product through the column-major library: C^T = B^T A^T, where a row-major [r,c] array is the
-// column-major [c,r] one.
-int gemm_rm(rocblas_handle h, Layout layout, int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-            float beta, int dtype) {
-    const rocblas_datatype dt = dtype == FMOE_F32 ? rocblas_datatype_f32_r : (dtype == FMOE_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f16_r);
-    const float alpha = 1.0f;
-    const rocblas_status st = api().gemm_ex(h, rocblas_operation_none, layout == kNN ? rocblas_operation_none : rocblas_operation_transpose,
-                                            N, M, K, &alpha, B, dt, ldb, A, dt, lda, &beta, C, dt, ldc, C, dt, ldc,
-                                            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
-    FMOE_REQUIRE(st == rocblas_status_success, FMOE_ERR_LIBRARY, "fmoe_mlp_backward: rocblas_gemm_ex failed (%d)", (int)st);
-    return FMOE_OK;
-}
+constexpr int kNN = kBlasNN, kTN = kBlasTN;
 
 struct MlpBwdPlan {
     size_t off_a, off_b, off_dh, off_h, off_dab, bytes;
@@ -100,6 +87,24 @@ MlpBwdPlan plan_mlp_backward(int64_t T_, int I, int dtype) {
 }
 
 }  // namespace
+
+// Row-major product through the column-major library: C^T = B^T A^T, where a row-major [r,c] array is the
+// column-major [c,r] one.  fp32 accumulation; A, B and C have the element type `dtype`.
+int blas_gemm(int layout, int M, int N, int K, const void* A, int lda, const void* B, int ldb, void* C, int ldc, float beta,
+              int dtype, hipStream_t stream) {
+    std::lock_guard<std::mutex> guard(api().lock);
+    rocblas_handle h = nullptr;
+    if (int rc = rocblas_for_device(&h)) return rc;
+    FMOE_REQUIRE(api().set_stream(h, stream) == rocblas_status_success, FMOE_ERR_LIBRARY, "rocblas_set_stream failed");
+    const rocblas_datatype dt = dtype == FMOE_F32 ? rocblas_datatype_f32_r : (dtype == FMOE_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f16_r);
+    const float alpha = 1.0f;
+    const rocblas_status st = api().gemm_ex(h, rocblas_operation_none, layout == kBlasNN ? rocblas_operation_none : rocblas_operation_transpose,
+                                            N, M, K, &alpha, B, dt, ldb, A, dt, lda, &beta, C, dt, ldc, C, dt, ldc,
+                                            rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    FMOE_REQUIRE(st == rocblas_status_success, FMOE_ERR_LIBRARY, "rocblas_gemm_ex failed (%d)", (int)st);
+    return FMOE_OK;
+}
+
 }  // namespace fmoe
 
 extern "C" size_t fmoe_mlp_backward_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int dtype) {
@@ -144,23 +149,17 @@ extern "C" int fmoe_mlp_backward(const void* dy, const void* x, const void* gate
         if (rc) return rc;
     }
 
-    std::lock_guard<std::mutex> guard(api().lock);
-    rocblas_handle handle = nullptr;
-    rc = rocblas_for_device(&handle);
-    if (rc) return rc;
-    FMOE_REQUIRE(api().set_stream(handle, s) == rocblas_status_success, FMOE_ERR_LIBRARY, "fmoe_mlp_backward: rocblas_set_stream failed");
-
-    rc = gemm_rm(handle, kNN, T_, I, H, dy, H, down_w, I, dh, I, 0.0f, dtype);                        // dh = dy Wd
+    rc = blas_gemm(kNN, T_, I, H, dy, H, down_w, I, dh, I, 0.0f, dtype, s);                        // dh = dy Wd
     if (rc) return rc;
     rc = launch_swiglu_backward(dh, a, b, dab, dab + (size_t)I * elt, h, num_tokens, I, 2 * (int64_t)I, 2 * (int64_t)I, dtype, s);
     if (rc) return rc;
-    rc = gemm_rm(handle, kTN, H, I, T_, dy, H, h, I, ddown_w, I, 0.0f, dtype);                         // dWd = dy^T h
+    rc = blas_gemm(kTN, H, I, T_, dy, H, h, I, ddown_w, I, 0.0f, dtype, s);                         // dWd = dy^T h
     if (rc) return rc;
-    rc = gemm_rm(handle, kNN, T_, H, I, dab, 2 * I, gate_w, H, dx, H, 0.0f, dtype);                    // dx = da Wg
+    rc = blas_gemm(kNN, T_, H, I, dab, 2 * I, gate_w, H, dx, H, 0.0f, dtype, s);                    // dx = da Wg
     if (rc) return rc;
-    rc = gemm_rm(handle, kNN, T_, H, I, dab + (size_t)I * elt, 2 * I, up_w, H, dx, H, 1.0f, dtype);    //    + db Wu
+    rc = blas_gemm(kNN, T_, H, I, dab + (size_t)I * elt, 2 * I, up_w, H, dx, H, 1.0f, dtype, s);    //    + db Wu
     if (rc) return rc;
-    rc = gemm_rm(handle, kTN, I, H, T_, dab, 2 * I, x, H, dgate_w, H, 0.0f, dtype);                    // dWg = da^T x
+    rc = blas_gemm(kTN, I, H, T_, dab, 2 * I, x, H, dgate_w, H, 0.0f, dtype, s);                    // dWg = da^T x
     if (rc) return rc;
-    return gemm_rm(handle, kTN, I, H, T_, dab + (size_t)I * elt, 2 * I, x, H, dup_w, H, 0.0f, dtype);  // dWu = db^T x
+    return blas_gemm(kTN, I, H, T_, dab + (size_t)I * elt, 2 * I, x, H, dup_w, H, 0.0f, dtype, s);  // dWu = db^T x
 }

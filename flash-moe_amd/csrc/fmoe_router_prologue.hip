@@ -16,34 +16,13 @@
 
 #include "fmoe_common.h"
 #include "fmoe_mfma.h"
+#include "fmoe_vec.h"
 
 namespace fmoe {
 namespace {
 
 constexpr int kStatsThreads = 256;
 constexpr int kMaxRowBlocks = 256;
-
-template <typename T> __device__ inline void unpack16(u32x4_t raw, float* v);
-template <> __device__ inline void unpack16<float>(u32x4_t raw, float* v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(raw[i]);
-}
-template <> __device__ inline void unpack16<bf16_t>(u32x4_t raw, float* v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        v[2 * i] = __uint_as_float(raw[i] << 16);
-        v[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
-    }
-}
-template <> __device__ inline void unpack16<f16_t>(u32x4_t raw, float* v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t w = raw[i];
-        const f16x2_t p = __builtin_bit_cast(f16x2_t, w);
-        v[2 * i] = (float)p[0];
-        v[2 * i + 1] = (float)p[1];
-    }
-}
 
 // Block (rb, strip): rows [rb*rows_per_block, ...), columns strip*64*V + lane*V .. +V; the 4 waves take rows 4 apart.
 // Sums are taken relative to the block's first row (pivot) so that var = E[d^2] - E[d]^2 does not cancel.
@@ -387,6 +366,173 @@ void launch_finalize(const float* partial, const ProloguePlan& p, int H, int tra
                        p.row_blocks, H, training, momentum, eps, rm, rv, nbt, mean_rstd);
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Backward of the prologue (batch norm + gate product), for the differentiable composition of the block.
+//   d   = dlogits (fp32) rounded to the activation dtype          q = round((x - mean) * rstd)     [recomputed]
+//   dWr = d^T q,  dq = d Wr                                        (library GEMMs)
+//   dx  = rstd * (dq - mean_t(dq) - xhat * mean_t(dq * xhat))      (training; xhat unrounded)   |   rstd * dq  (evaluation)
+// ------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void prologue_bwd_prepare_kernel(const float* __restrict__ dlogits, const T* __restrict__ x,
+                                                                  const float* __restrict__ mean_rstd, T* __restrict__ d16,
+                                                                  T* __restrict__ q, int64_t num_tokens, int hidden, int n_out) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t q_packets = num_tokens * (hidden / V), d_packets = num_tokens * (int64_t)n_out / V;
+    if (id < q_packets) {
+        const int col = (int)(id % (hidden / V)) * V;
+        float xv[V], qv[V];
+        unpack16<T>(reinterpret_cast<const u32x4_t*>(x)[id], xv);
+#pragma unroll
+        for (int v = 0; v < V; ++v) qv[v] = (xv[v] - mean_rstd[col + v]) * mean_rstd[hidden + col + v];
+        reinterpret_cast<u32x4_t*>(q)[id] = pack16<T>(qv);
+    } else if (id < q_packets + d_packets) {
+        const int64_t j = id - q_packets;
+        float dv[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) dv[v] = dlogits[j * V + v];
+        reinterpret_cast<u32x4_t*>(d16)[j] = pack16<T>(dv);
+    }
+}
+
+// partial: [row_blocks][2][H] = (sum dq, sum dq * xhat) over the block's rows; same geometry as bn_partial_kernel.
+template <typename T>
+__global__ __launch_bounds__(kStatsThreads) void bn_bwd_partial_kernel(const T* __restrict__ x, const T* __restrict__ dq,
+                                                                      const float* __restrict__ mean_rstd, int64_t num_tokens,
+                                                                      int hidden, int rows_per_block, float* __restrict__ partial) {
+    constexpr int V = Elem<T>::kVec;
+    __shared__ float red[3][2][kWave * V];
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int col = ((int)blockIdx.y * kWave + lane) * V;
+    const bool col_ok = col < hidden;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < num_tokens ? r0 + rows_per_block : num_tokens;
+    float mean[V], rstd[V], s1[V], s2[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        mean[v] = col_ok ? mean_rstd[col + v] : 0.0f;
+        rstd[v] = col_ok ? mean_rstd[hidden + col + v] : 0.0f;
+        s1[v] = s2[v] = 0.0f;
+    }
+    if (col_ok) {
+        for (int64_t r = r0 + wave; r < r1; r += 4) {
+            float xv[V], gv[V];
+            unpack16<T>(*reinterpret_cast<const u32x4_t*>(x + r * hidden + col), xv);
+            unpack16<T>(*reinterpret_cast<const u32x4_t*>(dq + r * hidden + col), gv);
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                s1[v] += gv[v];
+                s2[v] = __builtin_fmaf(gv[v], (xv[v] - mean[v]) * rstd[v], s2[v]);
+            }
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            red[wave - 1][0][lane * V + v] = s1[v];
+            red[wave - 1][1][lane * V + v] = s2[v];
+        }
+    }
+    __syncthreads();
+    if (wave == 0 && col_ok) {
+        float* out = partial + (int64_t)blockIdx.x * 2 * hidden;
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            float a = s1[v], b = s2[v];
+#pragma unroll
+            for (int w = 0; w < 3; ++w) {
+                a += red[w][0][lane * V + v];
+                b += red[w][1][lane * V + v];
+            }
+            out[col + v] = a;
+            out[hidden + col + v] = b;
+        }
+    }
+}
+
+// sums[0][c] = sum over row blocks of partial[.][0][c] / T, sums[1][c] likewise: the two column means of the formula
+__global__ __launch_bounds__(256) void bn_bwd_finalize_kernel(const float* __restrict__ partial, int row_blocks, int hidden,
+                                                              float inv_tokens, float* __restrict__ sums) {
+    const int c = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (c >= 2 * hidden) return;
+    float a = 0.0f;
+    for (int b = 0; b < row_blocks; ++b) a += partial[(int64_t)b * 2 * hidden + c];
+    sums[c] = a * inv_tokens;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__ x, const T* __restrict__ dq,
+                                                           const float* __restrict__ mean_rstd, const float* __restrict__ sums,
+                                                           T* __restrict__ dx, int64_t num_tokens, int hidden, int training) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= num_tokens * (hidden / V)) return;
+    const int col = (int)(id % (hidden / V)) * V;
+    float xv[V], gv[V], ov[V];
+    unpack16<T>(reinterpret_cast<const u32x4_t*>(x)[id], xv);
+    unpack16<T>(reinterpret_cast<const u32x4_t*>(dq)[id], gv);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const float rstd = mean_rstd[hidden + col + v];
+        if (training) {
+            const float xhat = (xv[v] - mean_rstd[col + v]) * rstd;
+            ov[v] = rstd * (gv[v] - sums[col + v] - xhat * sums[hidden + col + v]);
+        } else {
+            ov[v] = rstd * gv[v];
+        }
+    }
+    reinterpret_cast<u32x4_t*>(dx)[id] = pack16<T>(ov);
+}
+
+struct PrologueBwdPlan {
+    size_t off_d16, off_q, off_dq, off_partial, off_sums, bytes;
+};
+
+PrologueBwdPlan plan_prologue_backward(int64_t T_, int H, int nk, int dtype) {
+    PrologueBwdPlan p;
+    const size_t elt = dtype_size(dtype);
+    size_t o = 0;
+    auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
+    p.off_d16 = take((size_t)T_ * 2 * nk * elt);
+    p.off_q = take((size_t)T_ * H * elt);
+    p.off_dq = take((size_t)T_ * H * elt);
+    p.off_partial = take((size_t)kMaxRowBlocks * 2 * H * 4);
+    p.off_sums = take((size_t)2 * H * 4);
+    p.bytes = o;
+    return p;
+}
+
+template <typename T>
+int launch_prologue_backward(const float* dlogits, const void* x, const void* gate_w, const float* mean_rstd, int training,
+                             int64_t T_, int H, int nk, int dtype, void* dx, void* dgate_w, void* workspace, hipStream_t s) {
+    constexpr int V = Elem<T>::kVec;
+    const PrologueBwdPlan p = plan_prologue_backward(T_, H, nk, dtype);
+    const ProloguePlan rows = plan_prologue(T_, H, nk);
+    char* ws = (char*)workspace;
+    T *d16 = (T*)(ws + p.off_d16), *q = (T*)(ws + p.off_q), *dq = (T*)(ws + p.off_dq);
+    float *partial = (float*)(ws + p.off_partial), *sums = (float*)(ws + p.off_sums);
+    const int N = 2 * nk;
+    const int64_t packets = T_ * (H / V) + T_ * (int64_t)N / V;
+    hipLaunchKernelGGL((prologue_bwd_prepare_kernel<T>), dim3((unsigned)((packets + 255) / 256)), dim3(256), 0, s, dlogits,
+                       (const T*)x, mean_rstd, d16, q, T_, H, N);
+    FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(prepare)");
+    if (int rc = blas_gemm(kBlasTN, N, H, (int)T_, d16, N, q, H, dgate_w, H, 0.0f, dtype, s)) return rc;      // dWr = d^T q
+    if (int rc = blas_gemm(kBlasNN, (int)T_, H, N, d16, N, gate_w, H, dq, H, 0.0f, dtype, s)) return rc;       // dq = d Wr
+    if (training) {
+        const int strips = (H + kWave * V - 1) / (kWave * V);
+        hipLaunchKernelGGL((bn_bwd_partial_kernel<T>), dim3((unsigned)rows.row_blocks, (unsigned)strips), dim3(kStatsThreads), 0, s,
+                           (const T*)x, (const T*)dq, mean_rstd, T_, H, rows.rows_per_block, partial);
+        FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(column sums)");
+        hipLaunchKernelGGL(bn_bwd_finalize_kernel, dim3((unsigned)((2 * H + 255) / 256)), dim3(256), 0, s, (const float*)partial,
+                           rows.row_blocks, H, 1.0f / (float)T_, sums);
+        FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(finalize)");
+    }
+    hipLaunchKernelGGL((bn_bwd_apply_kernel<T>), dim3((unsigned)((T_ * (H / V) + 255) / 256)), dim3(256), 0, s, (const T*)x,
+                       (const T*)dq, mean_rstd, (const float*)sums, (T*)dx, T_, H, training);
+    FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(apply)");
+    return FMOE_OK;
+}
+
 }  // namespace
 }  // namespace fmoe
 
@@ -479,4 +625,40 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
     if (top_k == 0) return FMOE_OK;
     return launch_router_from_logits(logits32, num_tokens, num_keys, top_k, scores, indices, gates, dtype, norm_topk_prob,
                                      row_offsets, row_bytes, s);
+}
+
+extern "C" size_t fmoe_router_workspace_stats_offset(int64_t num_tokens, int hidden, int num_keys) {
+    if (num_tokens <= 0 || hidden <= 0 || num_keys <= 0) return 0;
+    return fmoe::plan_prologue(num_tokens, hidden, num_keys).off_mean_rstd;
+}
+
+extern "C" size_t fmoe_router_prologue_backward_workspace_bytes(int64_t num_tokens, int hidden, int num_keys, int dtype) {
+    if (num_tokens <= 0 || hidden <= 0 || num_keys <= 0 || !fmoe::dtype_ok(dtype)) return 0;
+    return fmoe::plan_prologue_backward(num_tokens, hidden, num_keys, dtype).bytes;
+}
+
+extern "C" int fmoe_router_prologue_backward(const float* dlogits_fp32, const void* x, const void* gate_w, const float* mean_rstd,
+                                             int training, int64_t num_tokens, int hidden, int num_keys, int dtype, void* dx,
+                                             void* dgate_w, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_router_prologue_backward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(num_tokens > 0 && hidden > 0 && num_keys > 0 && num_tokens < (1ll << 31), FMOE_ERR_BAD_SHAPE,
+                 "fmoe_router_prologue_backward: bad shape T=%lld H=%d nk=%d", (long long)num_tokens, hidden, num_keys);
+    const int vec = (int)(16 / dtype_size(dtype));
+    FMOE_REQUIRE(hidden % vec == 0 && (2 * num_keys) % vec == 0, FMOE_ERR_ALIGNMENT,
+                 "fmoe_router_prologue_backward: hidden=%d and 2*num_keys=%d must be multiples of %d", hidden, 2 * num_keys, vec);
+    FMOE_REQUIRE(dlogits_fp32 && x && gate_w && mean_rstd && dx && dgate_w, FMOE_ERR_NULL_POINTER,
+                 "fmoe_router_prologue_backward: null tensor pointer");
+    FMOE_REQUIRE(aligned16(x) && aligned16(dx) && aligned16(dlogits_fp32), FMOE_ERR_ALIGNMENT,
+                 "fmoe_router_prologue_backward: tensor pointers must be 16-byte aligned");
+    const size_t need = plan_prologue_backward(num_tokens, hidden, num_keys, dtype).bytes;
+    FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
+                 "fmoe_router_prologue_backward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FMOE_F32: return launch_prologue_backward<float>(dlogits_fp32, x, gate_w, mean_rstd, training, num_tokens, hidden, num_keys, dtype, dx, dgate_w, workspace, s);
+        case FMOE_BF16: return launch_prologue_backward<bf16_t>(dlogits_fp32, x, gate_w, mean_rstd, training, num_tokens, hidden, num_keys, dtype, dx, dgate_w, workspace, s);
+        default: return launch_prologue_backward<f16_t>(dlogits_fp32, x, gate_w, mean_rstd, training, num_tokens, hidden, num_keys, dtype, dx, dgate_w, workspace, s);
+    }
 }

@@ -79,4 +79,27 @@ template <> __device__ inline u32x4_t pack16<f16_t>(const float* v) {
     return r;
 }
 
+// the elements of a packet as fp32
+template <typename T> __device__ inline void unpack16(u32x4_t w, float* v);
+template <> __device__ inline void unpack16<float>(u32x4_t w, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(w[i]);
+}
+template <> __device__ inline void unpack16<bf16_t>(u32x4_t w, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+template <> __device__ inline void unpack16<f16_t>(u32x4_t w, float* v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t wi = w[i];
+        const f16x2_t p = __builtin_bit_cast(f16x2_t, wi);
+        v[2 * i] = (float)p[0];
+        v[2 * i + 1] = (float)p[1];
+    }
+}
+
 }  // namespace fmoe

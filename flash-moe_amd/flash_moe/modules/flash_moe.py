@@ -11,8 +11,8 @@ pair (:55-105).
   shared SwiGLU MLP + add                                           ``fmoe_mlp_forward`` (the add is the second
                                                                     GEMM's epilogue)
 ``forward_staged`` runs the same three stages as three calls.  When gradients are being recorded ``forward`` takes
-``forward_autograd`` instead: the reference's own composition (torch batch norm, linear and log-softmax, then the router,
-expert and MLP ops, flash_moe/modules/flash_moe.py:62-101), whose three ops carry HIP backward passes.
+``forward_autograd`` instead: the reference's own composition (batch norm + router gate, log-softmax, then the router,
+expert and MLP ops, flash_moe/modules/flash_moe.py:62-101); every stage but the log-softmax carries a HIP backward pass.
 
 Routing is evaluated in fp32 whatever the module dtype: the normalised activations are rounded to the
 module dtype exactly as the reference does, but their product with the router gate, the log-softmax
@@ -32,7 +32,7 @@ import torch.nn.functional as F
 from flash_moe.ops.hip.flash_block import block_forward
 from flash_moe.ops.hip.flash_expert import expert_forward, flash_expert_func
 from flash_moe.ops.hip.flash_mlp import flash_mlp_func, mlp_forward
-from flash_moe.ops.hip.flash_router import flash_router_func, router_forward
+from flash_moe.ops.hip.flash_router import flash_router_func, router_forward, router_prologue
 
 _SILU_NAMES = ("silu", "swish")
 
@@ -105,9 +105,12 @@ class FlashMoE(nn.Module):
         bsz, seq_len, _ = hidden_states.shape
         tokens = hidden_states.reshape(bsz * seq_len, self.hidden_size)
         num_tokens = tokens.shape[0]
-        query = self.router_norm(tokens)
-        logits32 = F.linear(query.float(), self.router_gate.weight.float())
-        router_logits = logits32.to(tokens.dtype).view(num_tokens, 2, self.num_keys).transpose(0, 1)
+        if num_tokens == 0:
+            logits32 = F.linear(self.router_norm(tokens).float(), self.router_gate.weight.float())
+            logits = logits32.to(tokens.dtype)
+        else:
+            logits32, logits = router_prologue(tokens, self.router_gate.weight, self.router_norm)
+        router_logits = logits.view(num_tokens, 2, self.num_keys).transpose(0, 1)
         log_probs = F.log_softmax(logits32.view(num_tokens, 2, self.num_keys), dim=-1).transpose(0, 1)
         scores, indices = flash_router_func(log_probs, self.num_keys, self.top_k)
         gates = torch.exp(scores)

@@ -109,6 +109,68 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
     return logits, scores, indices, gates
 
 
+class RouterPrologueFunc(torch.autograd.Function):
+    """Differentiable router prologue ``logits = BatchNorm1d(x) @ gate_weight.T`` (flash_moe/modules/flash_moe.py:62-67).
+
+    Forward: the batch-norm and gate launches of ``fmoe_router_forward`` (top_k = 0); returns the fp32 logits the routing
+    is computed from and their rounding to the activation dtype (what the module returns).  Backward:
+    ``fmoe_router_prologue_backward``.  ``norm``'s running statistics are updated in training mode, as by any forward."""
+
+    @staticmethod
+    def forward(ctx, tokens, gate_weight, norm):
+        num_expert_keys = gate_weight.shape[0] // 2
+        dev, training = check_router_args(tokens, gate_weight, norm, num_expert_keys, 0)
+        x, w = tokens.contiguous(), gate_weight.contiguous()
+        T, H = x.shape
+        logits = torch.empty((T, 2 * num_expert_keys), device=dev, dtype=x.dtype)
+        logits32 = torch.empty((T, 2 * num_expert_keys), device=dev, dtype=torch.float32)
+        L = _C.lib()
+        ws_bytes = L.fmoe_router_workspace_bytes(T, H, num_expert_keys)
+        ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+        rm, rv, nbt = norm.running_mean, norm.running_var, norm.num_batches_tracked
+        with torch.cuda.device(dev):
+            status = L.fmoe_router_forward(
+                _C.ptr(x), _C.ptr(w), _C.ptr(rm), _C.ptr(rv), _C.ptr(nbt), _C.dtype_code(rm.dtype), int(training),
+                float(norm.momentum), float(norm.eps), T, H, num_expert_keys, 0, _C.dtype_code(x.dtype), 0, _C.ptr(logits),
+                _C.ptr(logits32), None, None, None, _C.ptr(ws), ws_bytes, _C.current_stream(dev),
+            )
+        _C.check(status, "router prologue")
+        off = L.fmoe_router_workspace_stats_offset(T, H, num_expert_keys)
+        stats = ws[off:off + 2 * H * 4].view(torch.float32).clone()        # mean, 1/sqrt(var + eps): [2*H]
+        ctx.save_for_backward(x, w, stats)
+        ctx.training, ctx.num_expert_keys = training, num_expert_keys
+        return logits32, logits
+
+    @staticmethod
+    def backward(ctx, dlogits32, dlogits):
+        x, w, stats = ctx.saved_tensors
+        T, H = x.shape
+        grad = None
+        for g in (dlogits32, dlogits):
+            if g is not None:
+                grad = g.float() if grad is None else grad + g.float()
+        if grad is None:
+            return None, None, None
+        grad = grad.contiguous()
+        dev = x.device
+        code = _C.dtype_code(x.dtype)
+        dx, dw = torch.empty_like(x), torch.empty_like(w)
+        L = _C.lib()
+        ws_bytes = L.fmoe_router_prologue_backward_workspace_bytes(T, H, ctx.num_expert_keys, code)
+        ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+        with torch.cuda.device(dev):
+            status = L.fmoe_router_prologue_backward(_C.ptr(grad), _C.ptr(x), _C.ptr(w), _C.ptr(stats), int(ctx.training), T, H,
+                                                     ctx.num_expert_keys, code, _C.ptr(dx), _C.ptr(dw), _C.ptr(ws), ws_bytes,
+                                                     _C.current_stream(dev))
+        _C.check(status, "router prologue backward")
+        return dx, dw, None
+
+
+def router_prologue(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.nn.BatchNorm1d):
+    """``(logits_fp32 [T, 2*nk], logits [T, 2*nk] in tokens.dtype)``, differentiable with respect to tokens and gate_weight."""
+    return RouterPrologueFunc.apply(tokens, gate_weight, norm)
+
+
 def router_topk_backward(dscores: torch.Tensor, indices: torch.Tensor, num_expert_keys: int) -> torch.Tensor:
     """Scatter of ``dscores`` [T, K] onto the two halves' keys -> [2, T, nk] in ``dscores.dtype`` (``fmoe_router_topk_backward``)."""
     if dscores.dim() != 2 or indices.shape != dscores.shape or indices.dtype != torch.int64:

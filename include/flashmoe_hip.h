@@ -216,6 +216,18 @@ int fmoe_pkm_forward(const void* values, const void* routing_weights, const int6
 int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64_t num_tokens, int num_keys, int top_k,
                               int dtype, void* drouter_logits, void* stream);
 
+/* Backward of the router prologue q = BatchNorm1d(x), logits = q gate_w^T (flash_moe/modules/flash_moe.py:62-67; autograd of
+ * torch ops in the reference).  The forward is fmoe_router_forward with top_k = 0: it leaves mean and 1/sqrt(var+eps), [2,H]
+ * fp32, at byte offset fmoe_router_workspace_stats_offset() of its workspace; pass that as mean_rstd.
+ *   dlogits_fp32 [T, 2*nk] fp32 (rounded to dtype for the two GEMMs); dx [T,H], dgate_w [2*nk,H]: dtype.
+ * training != 0: batch statistics were used (the gradient flows through mean and variance); else running statistics
+ * (constants).  The two GEMMs are rocBLAS calls. */
+size_t fmoe_router_workspace_stats_offset(int64_t num_tokens, int hidden, int num_keys);
+size_t fmoe_router_prologue_backward_workspace_bytes(int64_t num_tokens, int hidden, int num_keys, int dtype);
+int fmoe_router_prologue_backward(const float* dlogits_fp32, const void* x, const void* gate_w, const float* mean_rstd,
+                                  int training, int64_t num_tokens, int hidden, int num_keys, int dtype, void* dx,
+                                  void* dgate_w, void* workspace, size_t workspace_bytes, void* stream);
+
 /* swiglu_backward / _swiglu_backward_kernel (flash_moe/ops/triton/flash_mlp.py:64-102, 126-150): for c = silu(a) * b,
  *   da = dc * (silu(a) * (1 - sigmoid(a)) + sigmoid(a)) * b,   db = dc * silu(a),   all [rows, cols] dtype. */
 int fmoe_swiglu_backward(const void* dc, const void* a, const void* b, int64_t rows, int cols, int dtype, void* da,

@@ -157,6 +157,16 @@ def test_backward_argument_checks():
     assert rb(a, a, 4, 9000, 2, _C.F32, a, None) == -5
     assert rb(a, None, 4, 8, 2, _C.F32, a, None) == -1
     assert rb(None, None, 0, 8, 2, _C.F32, None, None) == 0
+    off = lib.fmoe_router_workspace_stats_offset(64, 128, 16)
+    assert 0 < off < lib.fmoe_router_workspace_bytes(64, 128, 16) and off % 256 == 0
+    pneed = lib.fmoe_router_prologue_backward_workspace_bytes(64, 128, 16, _C.BF16)
+    assert pneed >= 64 * 32 * 2 + 2 * 64 * 128 * 2 and pneed % 256 == 0
+    pb = lib.fmoe_router_prologue_backward
+    assert pb(a, a, a, a, 1, 64, 128, 16, 4, a, a, a, pneed, None) == -4
+    assert pb(a, a, a, a, 1, 0, 128, 16, _C.BF16, a, a, a, pneed, None) == -2
+    assert pb(a, a, a, a, 1, 64, 124, 16, _C.BF16, a, a, a, pneed, None) == -6
+    assert pb(None, a, a, a, 1, 64, 128, 16, _C.BF16, a, a, a, pneed, None) == -1
+    assert pb(a, a, a, a, 1, 64, 128, 16, _C.BF16, a, a, a, pneed - 1, None) == -7
     sb = lib.fmoe_swiglu_backward
     assert sb(a, a, a, 4, 64, 7, a, a, None) == -4
     assert sb(a, a, a, 4, 0, _C.BF16, a, a, None) == -2

@@ -265,3 +265,37 @@ def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
     torch.testing.assert_close(saved[1].float(), x.float() @ wu.float().t(), rtol=tol, atol=tol)
     for a, b in zip(mlp_backward(dy, x, wg, wu, wd, saved), mlp_backward(dy, x, wg, wu, wd)):
         assert rel_fro(a, b) < (1e-6 if dtype == torch.float32 else 2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("training", [True, False])
+@pytest.mark.parametrize("T,H,nk", [(256, 128, 16), (1000, 1024, 128), (65, 64, 8)])
+def test_router_prologue_backward(dtype, training, T, H, nk):
+    """Batch norm + gate product: gradients of the input and of the gate weights against float64 autograd."""
+    from flash_moe.ops.hip.flash_router import router_prologue
+
+    x = (torch.randn(T, H, generator=gen(1)) * 1.5 + 0.3).to(dtype)
+    w = (torch.randn(2 * nk, H, generator=gen(2)) * 0.05).to(dtype)
+    g32 = torch.randn(T, 2 * nk, generator=gen(3))
+    g16 = (torch.randn(T, 2 * nk, generator=gen(4)) * 0.5).to(dtype)
+    norm = torch.nn.BatchNorm1d(H, affine=False).cuda().to(dtype)
+    with torch.no_grad():
+        norm.running_mean.normal_(0.0, 0.2, generator=torch.Generator(device="cuda").manual_seed(5))
+        norm.running_var.uniform_(0.5, 2.0, generator=torch.Generator(device="cuda").manual_seed(6))
+    rm0, rv0 = norm.running_mean.clone(), norm.running_var.clone()
+    norm.train(training)
+    xd, wd = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    logits32, logits = router_prologue(xd, wd, norm)
+    assert logits32.dtype == torch.float32 and logits.dtype == dtype
+    ((logits32 * g32.cuda()).sum() + (logits.float() * g16.cuda().float()).sum()).backward()
+
+    x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    q = torch.nn.functional.batch_norm(x64, rm0.double().cpu(), rv0.double().cpu(), training=training, eps=1e-5)
+    ref = q @ w64.t()
+    (ref * (g32.double() + g16.double())).sum().backward()
+    tol = {torch.float32: 2e-5, torch.bfloat16: 1.2e-2, torch.float16: 3e-3}[dtype]
+    assert rel_fro(logits32, ref) < tol
+    assert rel_fro(xd.grad, x64.grad) < tol, f"dx {rel_fro(xd.grad, x64.grad):.3e}"
+    assert rel_fro(wd.grad, w64.grad) < tol, f"dgate {rel_fro(wd.grad, w64.grad):.3e}"
+    if training:   # a constant shift of the loss gradient along tokens cannot change dx: columns of dx sum to ~0
+        assert float(xd.grad.float().sum(0).abs().max()) < 50 * tol * float(xd.grad.float().abs().max()) * T ** 0.5
