@@ -72,19 +72,18 @@ int launch_router_backward(const void* dscores, const int64_t* indices, void* dl
 // ------------------------------------------------------------------------------------------------------------
 // SwiGLU
 // ------------------------------------------------------------------------------------------------------------
-// One 16-byte packet per thread.  Row strides (elements) let da / db / h live side by side in wider buffers.
+// One 16-byte packet per thread; workgroup b works on row b / col_blocks.  Row strides (elements) let da / db / h live
+// side by side in wider buffers.
 template <typename T>
 __global__ __launch_bounds__(256) void swiglu_backward_kernel(const T* __restrict__ dc, const T* __restrict__ a,
                                                               const T* __restrict__ b, T* __restrict__ da,
-                                                              T* __restrict__ db, T* __restrict__ h, int64_t rows,
+                                                              T* __restrict__ db, T* __restrict__ h, int col_blocks,
                                                               int cols, int64_t da_stride, int64_t db_stride) {
     constexpr int V = Elem<T>::kVec;
-    const int packets = cols / V;
-    const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (q >= rows * packets) return;
-    const int64_t row = q / packets;
-    const int col = (int)(q % packets) * V;
-    const int64_t at = row * cols + col;
+    const uint32_t row = blockIdx.x / (uint32_t)col_blocks;
+    const int col = ((int)(blockIdx.x % (uint32_t)col_blocks) * 256 + (int)threadIdx.x) * V;
+    if (col >= cols) return;
+    const int64_t at = (int64_t)row * cols + col;
     float dcv[V], av[V], bv[V], dav[V], dbv[V], hv[V];
     unpack16<T>(*reinterpret_cast<const u32x4_t*>(dc + at), dcv);
     unpack16<T>(*reinterpret_cast<const u32x4_t*>(a + at), av);
@@ -207,33 +206,44 @@ __global__ void zero_i32_kernel(int32_t* __restrict__ p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
 }
 
-// offsets[e] = number of pairs of experts < e, for e in [0, num_experts]; one workgroup, each thread owns a run of experts.
+// offsets[e] = number of pairs of experts < e, for e in [0, num_experts]; one workgroup.  The counts are taken in tiles
+// of kScanThreads * 4 (coalesced 16-byte loads, four counts per thread), each tile scanned across the workgroup with the
+// running total carried from tile to tile.
 constexpr int kScanThreads = 1024;
 __global__ __launch_bounds__(kScanThreads) void expert_scan_kernel(const int32_t* __restrict__ counts,
                                                                   int32_t* __restrict__ offsets, int64_t num_experts) {
     __shared__ int32_t wave_total[kScanThreads / kWave];
+    __shared__ int32_t carry_s;
     const int tid = (int)threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    const int64_t per = (num_experts + kScanThreads - 1) / kScanThreads;
-    const int64_t lo = (int64_t)tid * per, hi = lo + per < num_experts ? lo + per : num_experts;
-    int32_t mine = 0;
-    for (int64_t e = lo; e < hi; ++e) mine += counts[e];
-    // inclusive scan over the wave, then over the wave totals
-    int32_t incl = mine;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        const int32_t up = __shfl_up(incl, d, kWave);
-        if (lane >= d) incl += up;
-    }
-    if (lane == kWave - 1) wave_total[wave] = incl;
+    if (tid == 0) carry_s = 0;
     __syncthreads();
-    int32_t before = 0;
-    for (int w = 0; w < wave; ++w) before += wave_total[w];
-    int32_t run = before + incl - mine;
-    for (int64_t e = lo; e < hi; ++e) {
-        offsets[e] = run;
-        run += counts[e];
+    for (int64_t base = 0; base < num_experts; base += kScanThreads * 4) {
+        const int64_t e0 = base + (int64_t)tid * 4;
+        int32_t c[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = e0 + j < num_experts ? counts[e0 + j] : 0;
+        const int32_t mine = c[0] + c[1] + c[2] + c[3];
+        int32_t incl = mine;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const int32_t up = __shfl_up(incl, d, kWave);
+            if (lane >= d) incl += up;
+        }
+        if (lane == kWave - 1) wave_total[wave] = incl;
+        __syncthreads();
+        int32_t before = carry_s;
+        for (int w = 0; w < wave; ++w) before += wave_total[w];
+        int32_t run = before + incl - mine;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (e0 + j < num_experts) offsets[e0 + j] = run;
+            run += c[j];
+        }
+        __syncthreads();
+        if (tid == kScanThreads - 1) carry_s = run;      // the last thread's running total is the tile's inclusive total
+        __syncthreads();
     }
-    if (tid == kScanThreads - 1) offsets[num_experts] = before + incl;
+    if (tid == 0) offsets[num_experts] = carry_s;
 }
 
 // pairs[offsets[e] + (arrival order)] = p for every valid pair: segments are complete, their internal order is not fixed
@@ -429,21 +439,23 @@ __global__ void zero_fill_kernel(u32x4_t* __restrict__ p, size_t packets) {
 int launch_swiglu_backward(const void* dc, const void* a, const void* b, void* da, void* db, void* h, int64_t rows, int cols,
                            int64_t da_stride, int64_t db_stride, int dtype, hipStream_t stream) {
     const int vec = (int)(16 / dtype_size(dtype));
-    const int64_t packets = rows * (cols / vec);
-    if (packets == 0) return FMOE_OK;
-    const dim3 grid((unsigned)((packets + 255) / 256)), block(256);
+    if (rows == 0) return FMOE_OK;
+    const int col_blocks = (cols / vec + 255) / 256;
+    FMOE_REQUIRE(rows * col_blocks < (1ll << 31), FMOE_ERR_UNSUPPORTED, "fmoe_swiglu_backward: %lld rows of %d columns exceed the grid",
+                 (long long)rows, cols);
+    const dim3 grid((unsigned)(rows * col_blocks)), block(256);
     switch (dtype) {
         case FMOE_F32:
             hipLaunchKernelGGL((swiglu_backward_kernel<float>), grid, block, 0, stream, (const float*)dc, (const float*)a,
-                               (const float*)b, (float*)da, (float*)db, (float*)h, rows, cols, da_stride, db_stride);
+                               (const float*)b, (float*)da, (float*)db, (float*)h, col_blocks, cols, da_stride, db_stride);
             break;
         case FMOE_BF16:
             hipLaunchKernelGGL((swiglu_backward_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)dc, (const bf16_t*)a,
-                               (const bf16_t*)b, (bf16_t*)da, (bf16_t*)db, (bf16_t*)h, rows, cols, da_stride, db_stride);
+                               (const bf16_t*)b, (bf16_t*)da, (bf16_t*)db, (bf16_t*)h, col_blocks, cols, da_stride, db_stride);
             break;
         default:
             hipLaunchKernelGGL((swiglu_backward_kernel<f16_t>), grid, block, 0, stream, (const f16_t*)dc, (const f16_t*)a,
-                               (const f16_t*)b, (f16_t*)da, (f16_t*)db, (f16_t*)h, rows, cols, da_stride, db_stride);
+                               (const f16_t*)b, (f16_t*)da, (f16_t*)db, (f16_t*)h, col_blocks, cols, da_stride, db_stride);
     }
     FMOE_CHECK_LAUNCH("fmoe_swiglu_backward");
     return FMOE_OK;

@@ -372,26 +372,38 @@ void launch_finalize(const float* partial, const ProloguePlan& p, int H, int tra
 //   dWr = d^T q,  dq = d Wr                                        (library GEMMs)
 //   dx  = rstd * (dq - mean_t(dq) - xhat * mean_t(dq * xhat))      (training; xhat unrounded)   |   rstd * dq  (evaluation)
 // ------------------------------------------------------------------------------------------------------------
+// Workgroup b: row b / col_blocks of q (and of d), packets (b % col_blocks) * 256 + thread of that row.
 template <typename T>
 __global__ __launch_bounds__(256) void prologue_bwd_prepare_kernel(const float* __restrict__ dlogits, const T* __restrict__ x,
                                                                   const float* __restrict__ mean_rstd, T* __restrict__ d16,
-                                                                  T* __restrict__ q, int64_t num_tokens, int hidden, int n_out) {
+                                                                  T* __restrict__ q, int hidden, int n_out, int col_blocks) {
     constexpr int V = Elem<T>::kVec;
-    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t q_packets = num_tokens * (hidden / V), d_packets = num_tokens * (int64_t)n_out / V;
-    if (id < q_packets) {
-        const int col = (int)(id % (hidden / V)) * V;
+    const uint32_t row = blockIdx.x / (uint32_t)col_blocks;
+    const int pc = (int)(blockIdx.x % (uint32_t)col_blocks) * 256 + (int)threadIdx.x;
+    const int col = pc * V;
+    if (col < hidden) {
+        const int64_t at = (int64_t)row * hidden + col;
         float xv[V], qv[V];
-        unpack16<T>(reinterpret_cast<const u32x4_t*>(x)[id], xv);
+        unpack16<T>(*reinterpret_cast<const u32x4_t*>(x + at), xv);
 #pragma unroll
-        for (int v = 0; v < V; ++v) qv[v] = (xv[v] - mean_rstd[col + v]) * mean_rstd[hidden + col + v];
-        reinterpret_cast<u32x4_t*>(q)[id] = pack16<T>(qv);
-    } else if (id < q_packets + d_packets) {
-        const int64_t j = id - q_packets;
+        for (int h = 0; h < V / 4; ++h) {
+            const f32x4_t m = *reinterpret_cast<const f32x4_t*>(mean_rstd + col + 4 * h);
+            const f32x4_t r = *reinterpret_cast<const f32x4_t*>(mean_rstd + hidden + col + 4 * h);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) qv[4 * h + j] = (xv[4 * h + j] - m[j]) * r[j];
+        }
+        *reinterpret_cast<u32x4_t*>(q + at) = pack16<T>(qv);
+    }
+    if (col < n_out) {
+        const int64_t at = (int64_t)row * n_out + col;
         float dv[V];
 #pragma unroll
-        for (int v = 0; v < V; ++v) dv[v] = dlogits[j * V + v];
-        reinterpret_cast<u32x4_t*>(d16)[j] = pack16<T>(dv);
+        for (int h = 0; h < V / 4; ++h) {
+            const f32x4_t g = *reinterpret_cast<const f32x4_t*>(dlogits + at + 4 * h);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dv[4 * h + j] = g[j];
+        }
+        *reinterpret_cast<u32x4_t*>(d16 + at) = pack16<T>(dv);
     }
 }
 
@@ -450,38 +462,62 @@ __global__ __launch_bounds__(kStatsThreads) void bn_bwd_partial_kernel(const T* 
     }
 }
 
-// sums[0][c] = sum over row blocks of partial[.][0][c] / T, sums[1][c] likewise: the two column means of the formula
+// sums[0][c] = sum over row blocks of partial[.][0][c] / T, sums[1][c] likewise: the two column means of the formula.
+// The loads of 16 row blocks are issued together (independent accumulators), so a column costs a few memory round trips.
 __global__ __launch_bounds__(256) void bn_bwd_finalize_kernel(const float* __restrict__ partial, int row_blocks, int hidden,
                                                               float inv_tokens, float* __restrict__ sums) {
     const int c = (int)(blockIdx.x * blockDim.x + threadIdx.x);
     if (c >= 2 * hidden) return;
+    float acc[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) acc[u] = 0.0f;
+    for (int b0 = 0; b0 < row_blocks; b0 += 16) {
+        float got[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int b = b0 + u < row_blocks ? b0 + u : row_blocks - 1;      // clamped: every load is unconditional
+            got[u] = partial[(int64_t)b * 2 * hidden + c];
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc[u] += b0 + u < row_blocks ? got[u] : 0.0f;
+    }
     float a = 0.0f;
-    for (int b = 0; b < row_blocks; ++b) a += partial[(int64_t)b * 2 * hidden + c];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) a += acc[u];
     sums[c] = a * inv_tokens;
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__ x, const T* __restrict__ dq,
                                                            const float* __restrict__ mean_rstd, const float* __restrict__ sums,
-                                                           T* __restrict__ dx, int64_t num_tokens, int hidden, int training) {
+                                                           T* __restrict__ dx, int hidden, int col_blocks, int training) {
     constexpr int V = Elem<T>::kVec;
-    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (id >= num_tokens * (hidden / V)) return;
-    const int col = (int)(id % (hidden / V)) * V;
-    float xv[V], gv[V], ov[V];
-    unpack16<T>(reinterpret_cast<const u32x4_t*>(x)[id], xv);
-    unpack16<T>(reinterpret_cast<const u32x4_t*>(dq)[id], gv);
+    const uint32_t row = blockIdx.x / (uint32_t)col_blocks;
+    const int col = ((int)(blockIdx.x % (uint32_t)col_blocks) * 256 + (int)threadIdx.x) * V;
+    if (col >= hidden) return;
+    const int64_t at = (int64_t)row * hidden + col;
+    float xv[V], gv[V], ov[V], mean[V], rstd[V], m1[V], m2[V];
+    unpack16<T>(*reinterpret_cast<const u32x4_t*>(x + at), xv);
+    unpack16<T>(*reinterpret_cast<const u32x4_t*>(dq + at), gv);
+    // the four per-column vectors as 16-byte loads, all requested before any is used
 #pragma unroll
-    for (int v = 0; v < V; ++v) {
-        const float rstd = mean_rstd[hidden + col + v];
-        if (training) {
-            const float xhat = (xv[v] - mean_rstd[col + v]) * rstd;
-            ov[v] = rstd * (gv[v] - sums[col + v] - xhat * sums[hidden + col + v]);
-        } else {
-            ov[v] = rstd * gv[v];
+    for (int h = 0; h < V / 4; ++h) {
+        const f32x4_t a = *reinterpret_cast<const f32x4_t*>(mean_rstd + col + 4 * h);
+        const f32x4_t b = *reinterpret_cast<const f32x4_t*>(mean_rstd + hidden + col + 4 * h);
+        const f32x4_t c = training ? *reinterpret_cast<const f32x4_t*>(sums + col + 4 * h) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        const f32x4_t d = training ? *reinterpret_cast<const f32x4_t*>(sums + hidden + col + 4 * h) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            mean[4 * h + j] = a[j];
+            rstd[4 * h + j] = b[j];
+            m1[4 * h + j] = c[j];
+            m2[4 * h + j] = d[j];
         }
     }
-    reinterpret_cast<u32x4_t*>(dx)[id] = pack16<T>(ov);
+    // evaluation mode: m1 = m2 = 0 and the formula reduces to rstd * dq
+#pragma unroll
+    for (int v = 0; v < V; ++v) ov[v] = rstd[v] * (gv[v] - m1[v] - (xv[v] - mean[v]) * rstd[v] * m2[v]);
+    *reinterpret_cast<u32x4_t*>(dx + at) = pack16<T>(ov);
 }
 
 struct PrologueBwdPlan {
@@ -512,9 +548,10 @@ int launch_prologue_backward(const float* dlogits, const void* x, const void* ga
     T *d16 = (T*)(ws + p.off_d16), *q = (T*)(ws + p.off_q), *dq = (T*)(ws + p.off_dq);
     float *partial = (float*)(ws + p.off_partial), *sums = (float*)(ws + p.off_sums);
     const int N = 2 * nk;
-    const int64_t packets = T_ * (H / V) + T_ * (int64_t)N / V;
-    hipLaunchKernelGGL((prologue_bwd_prepare_kernel<T>), dim3((unsigned)((packets + 255) / 256)), dim3(256), 0, s, dlogits,
-                       (const T*)x, mean_rstd, d16, q, T_, H, N);
+    const int widest = H > N ? H : N;
+    const int col_blocks = (widest / V + 255) / 256;
+    hipLaunchKernelGGL((prologue_bwd_prepare_kernel<T>), dim3((unsigned)(T_ * col_blocks)), dim3(256), 0, s, dlogits,
+                       (const T*)x, mean_rstd, d16, q, H, N, col_blocks);
     FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(prepare)");
     if (int rc = blas_gemm(kBlasTN, N, H, (int)T_, d16, N, q, H, dgate_w, H, 0.0f, dtype, s)) return rc;      // dWr = d^T q
     if (int rc = blas_gemm(kBlasNN, (int)T_, H, N, d16, N, gate_w, H, dq, H, 0.0f, dtype, s)) return rc;       // dq = d Wr
@@ -527,8 +564,9 @@ int launch_prologue_backward(const float* dlogits, const void* x, const void* ga
                            rows.row_blocks, H, 1.0f / (float)T_, sums);
         FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(finalize)");
     }
-    hipLaunchKernelGGL((bn_bwd_apply_kernel<T>), dim3((unsigned)((T_ * (H / V) + 255) / 256)), dim3(256), 0, s, (const T*)x,
-                       (const T*)dq, mean_rstd, (const float*)sums, (T*)dx, T_, H, training);
+    const int apply_blocks = (H / V + 255) / 256;
+    hipLaunchKernelGGL((bn_bwd_apply_kernel<T>), dim3((unsigned)(T_ * apply_blocks)), dim3(256), 0, s, (const T*)x,
+                       (const T*)dq, mean_rstd, (const float*)sums, (T*)dx, H, apply_blocks, training);
     FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(apply)");
     return FMOE_OK;
 }
@@ -643,14 +681,14 @@ extern "C" int fmoe_router_prologue_backward(const float* dlogits_fp32, const vo
     using namespace fmoe;
     clear_error();
     FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_router_prologue_backward: unknown dtype %d", dtype);
-    FMOE_REQUIRE(num_tokens > 0 && hidden > 0 && num_keys > 0 && num_tokens < (1ll << 31), FMOE_ERR_BAD_SHAPE,
+    FMOE_REQUIRE(num_tokens > 0 && hidden > 0 && num_keys > 0 && num_tokens < (1ll << 24), FMOE_ERR_BAD_SHAPE,
                  "fmoe_router_prologue_backward: bad shape T=%lld H=%d nk=%d", (long long)num_tokens, hidden, num_keys);
     const int vec = (int)(16 / dtype_size(dtype));
     FMOE_REQUIRE(hidden % vec == 0 && (2 * num_keys) % vec == 0, FMOE_ERR_ALIGNMENT,
                  "fmoe_router_prologue_backward: hidden=%d and 2*num_keys=%d must be multiples of %d", hidden, 2 * num_keys, vec);
     FMOE_REQUIRE(dlogits_fp32 && x && gate_w && mean_rstd && dx && dgate_w, FMOE_ERR_NULL_POINTER,
                  "fmoe_router_prologue_backward: null tensor pointer");
-    FMOE_REQUIRE(aligned16(x) && aligned16(dx) && aligned16(dlogits_fp32), FMOE_ERR_ALIGNMENT,
+    FMOE_REQUIRE(aligned16(x) && aligned16(dx) && aligned16(dlogits_fp32) && aligned16(mean_rstd), FMOE_ERR_ALIGNMENT,
                  "fmoe_router_prologue_backward: tensor pointers must be 16-byte aligned");
     const size_t need = plan_prologue_backward(num_tokens, hidden, num_keys, dtype).bytes;
     FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
