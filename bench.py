@@ -349,8 +349,8 @@ def main():
                     help="also run a 256 MiB device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
-        print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (the forward path is single-GPU; "
-              "see DESIGN.md for how it would shard)", file=sys.stderr)
+        print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (the path is single-GPU: tokens would be "
+              "split across devices with one all-reduce of the batch-norm statistics, or the tables sharded by expert)", file=sys.stderr)
         sys.exit(2)
 
     import torch
