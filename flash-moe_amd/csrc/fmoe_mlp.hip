@@ -224,6 +224,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     const int lrow = lane / CPR, lp = lane % CPR;
     const int key_dma = ((wave * RPI + lrow) >> ROW_SHIFT) & (CPR - 1);
     const uint32_t lane_off = (uint32_t)(lrow * K + ((lp ^ key_dma) << 3)) * (uint32_t)sizeof(T);   // bytes
+    // A rows beyond M (a ragged last tile row) are read from row M-1 instead: one byte offset per DMA round, set per
+    // tile.  What the MFMAs make of those rows is never stored (the epilogue's buffer stores are bounds-checked).
+    uint32_t a_lane_off[A_ROUNDS];
     const T *a_src, *b_src0, *b_src1 = nullptr;
     int m0, n0;
     // The workgroup is persistent: it takes tiles t, t + gridDim.x, ...  Each XCD (workgroup id mod 8) gets a contiguous
@@ -235,7 +238,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
         m0 = (first_m + (t % width) % gsz) * BM;
         n0 = ((t % width) / gsz) * BN_OUT;
-        a_src = A + (int64_t)(m0 + wave * RPI) * K;      // wave-uniform; the lane's part is the 32-bit lane_off
+        a_src = A + (int64_t)m0 * K;                     // wave-uniform; the lane's part is the 32-bit a_lane_off[r]
+#pragma unroll
+        for (int r = 0; r < A_ROUNDS; ++r) {
+            int row = r * ROWS_PER_IT + wave * RPI + lrow;
+            row = m0 + row < M ? row : M - 1 - m0;
+            a_lane_off[r] = (uint32_t)(row * K + ((lp ^ key_dma) << 3)) * (uint32_t)sizeof(T);
+        }
         b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K;
         if (EPI == kEpiSwiGLU) b_src1 = B1 + (int64_t)(n0 + wave * RPI) * K;
     };
@@ -244,7 +253,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
         for (int r = 0; r < A_ROUNDS; ++r)
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)((const char*)(a_src + (int64_t)r * ROWS_PER_IT * K + k0) + lane_off),
+                (const __attribute__((address_space(1))) void*)((const char*)(a_src + k0) + a_lane_off[r]),
                 (__attribute__((address_space(3))) void*)(stage + (r * ROWS_PER_IT + wave * RPI) * BKT), 16, 0, 0);
 #pragma unroll
         for (int r = 0; r < B_ROUNDS; ++r) {
@@ -343,11 +352,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
                 for (int i = 0; i < MF; ++i)
 #pragma unroll
                     for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks % RING][i], fb[ks % RING][j], acc[i][j]);
-                static_assert(kReads <= kMfmas, "one LDS read after each of the first MFMAs");
+                // issue order: the LDS reads spread evenly behind the MFMAs
+                constexpr int kPer = (kReads + kMfmas - 1) / kMfmas;
 #pragma unroll
                 for (int q = 0; q < kMfmas; ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    if (reads && q < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (reads && q * kPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
                 }
             }
         };
@@ -373,7 +383,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         const int lane_bytes = ((4 * fhalf) * N + frow) * (int)sizeof(T);
         const int64_t wave_off = (int64_t)(out_m0 + wm * WM) * N + out_n0 + wn * ((EPI == kEpiSwiGLU) ? WN / 2 : WN);
         const int64_t span = ((int64_t)M * N - wave_off) * (int64_t)sizeof(T);
-        const int span32 = (int)(span < 0x7FFFFFFFll ? span : 0x7FFFFFFFll);
+        // a wave whose rows all lie beyond M gets an empty descriptor: every access of it is dropped
+        const int span32 = (int)(span < 0 ? 0 : (span < 0x7FFFFFFFll ? span : 0x7FFFFFFFll));
         auto c_rsrc = __builtin_amdgcn_make_buffer_rsrc(C + wave_off, 0, span32, 0x00020000);
         auto store_elem = [&](int uni_bytes, float value) {
             const T t = Elem<T>::from_f32(value);
@@ -499,7 +510,7 @@ void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
 void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
-    const int tiles_m = M / BM, tiles_n = N / BN_OUT;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = N / BN_OUT;      // a ragged last row of tiles is allowed
     // persistent workgroups: as many as are resident at once (LDS-limited), a multiple of 8 so that the XCD patches hold
     constexpr int kStageBytes = (BM + BN) * BKT * (int)sizeof(T) * NSTAGE;
     constexpr int kPerCu = (160 * 1024 / kStageBytes) < 1 ? 1 : ((160 * 1024 / kStageBytes) > 2 ? 2 : (160 * 1024 / kStageBytes));
@@ -520,14 +531,26 @@ void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, 
     else launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
 }
 
+// Few tokens: 64-row tiles (wave tiles of 32 x 64 or 32 x 32), so that a batch of a few hundred tokens still gives
+// every CU a tile.  N_OUT: output columns of a tile.
+template <typename T, int EPI>
+void launch_narrow_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
+    if (EPI == kEpiPlain && (int64_t)((M + 63) / 64) * (N / 128) < 256 && N % 64 == 0)
+        launch_gemm_dma<T, 64, 64, 2, 2, 64, 4, kEpiPlain, 3>(A, B0, B1, C, R, M, N, K, stream);
+    else
+        launch_gemm_dma<T, 64, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+}
+
 template <typename T>
 int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
     const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu, *S = (const T*)saved;
     const bool k_ok = H % 64 == 0;
-    if (k_ok && M % 256 == 0 && I % 128 == 0 && (int64_t)(M / 256) * (I / 128) >= 256)
+    if (k_ok && I % 128 == 0 && (int64_t)((M + 255) / 256) * (I / 128) >= 256)
         launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, S, M, I, H, stream);
-    else if (k_ok && M % 128 == 0 && I % 64 == 0)
-        launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, (int64_t)(M / 128) * (I / 64), stream);
+    else if (k_ok && I % 64 == 0 && (int64_t)((M + 127) / 128) * (I / 64) >= 256)
+        launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, (int64_t)((M + 127) / 128) * (I / 64), stream);
+    else if (k_ok && I % 64 == 0)
+        launch_narrow_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
     else
         launch_gemm<T, 128, 128, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up)");
@@ -538,10 +561,12 @@ template <typename T>
 int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
     const T *A = (const T*)h, *W = (const T*)wd, *R = (const T*)residual;
     const bool k_ok = I % 64 == 0;
-    if (k_ok && M % 256 == 0 && H % 256 == 0 && (int64_t)(M / 256) * (H / 256) >= 256)
+    if (k_ok && H % 256 == 0 && (int64_t)((M + 255) / 256) * (H / 256) >= 256)
         launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiPlain, 1>(A, W, nullptr, (T*)out, R, M, H, I, stream);
-    else if (k_ok && M % 128 == 0 && H % 128 == 0)
-        launch_small_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, (int64_t)(M / 128) * (H / 128), stream);
+    else if (k_ok && H % 128 == 0 && (int64_t)((M + 127) / 128) * (H / 128) >= 256)
+        launch_small_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, (int64_t)((M + 127) / 128) * (H / 128), stream);
+    else if (k_ok && H % 128 == 0)
+        launch_narrow_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     else
         launch_gemm<T, 128, 128, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(down)");

@@ -26,6 +26,9 @@ def truth64(x, wg, wu, wd):
     (512, 256, 1024),      # C1
     (1024, 1024, 4096),    # C4 weights, fewer tokens (small-tile path)
     (4096, 1024, 4096),    # C4 (large-tile path for gate/up)
+    (192, 128, 256),       # 64-row tiles (T a multiple of 64 only)
+    (100, 128, 256),       # ragged T on the tiled path: the last tile row reads clamped rows, stores are bounds-checked
+    (1000, 256, 512),
     (200, 72, 136),        # ragged in every dimension
     (1, 64, 64),
 ])
