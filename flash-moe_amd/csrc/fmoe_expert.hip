@@ -27,15 +27,21 @@ constexpr int kPairsInFlight = 4;   // (down,up) row pairs requested ahead per w
 constexpr int kWavesPerBlock = 4;
 
 // NCH = number of 16-byte packets each lane holds per row: a row has at most NCH*64 packets.
-template <typename T, int NCH, int ACT>
+// SPLIT = false: one wave per token, kWavesPerBlock tokens per workgroup.  SPLIT = true (few tokens): the workgroup's
+// waves share one token, wave w taking pairs w*P .. w*P+P-1, (w+4)*P .. of it (P = pairs in flight), and their partial rows
+// are added in wave order through LDS: four times shorter dependency chains when there are not enough tokens to fill the
+// chip with one wave each.
+template <typename T, int NCH, int ACT, bool SPLIT>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
     const T* __restrict__ x, const T* __restrict__ down, const T* __restrict__ up,
     const int64_t* __restrict__ indices, const T* __restrict__ gates, T* __restrict__ out,
     int64_t num_tokens, int hidden, int64_t num_experts, int top_k) {
     constexpr int V = Elem<T>::kVec;
     const int lane = lane_id();
-    const int64_t token = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    if (token >= num_tokens) return;   // whole wave leaves together
+    const int wave = (int)(threadIdx.x >> 6);
+    const int64_t token = SPLIT ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * kWavesPerBlock + wave;
+    if (token >= num_tokens) return;   // whole wave leaves together (SPLIT: the whole workgroup)
+    __shared__ float partial_rows[SPLIT ? (kWavesPerBlock - 1) * NCH * V * kWave : 1];
 
     const int packets = hidden / V;   // 16-byte packets per row (hidden % V == 0 is checked on the host)
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
@@ -58,7 +64,9 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
     const int64_t* my_idx = indices + token * top_k;
     const T* my_gate = gates + token * top_k;
 
-    for (int k0 = 0; k0 < top_k; k0 += kPairsInFlight) {
+    const int k_first = SPLIT ? wave * kPairsInFlight : 0;
+    const int k_step = SPLIT ? kWavesPerBlock * kPairsInFlight : kPairsInFlight;
+    for (int k0 = k_first; k0 < top_k; k0 += k_step) {
         u32x4_t dn[kPairsInFlight][NCH];
         u32x4_t uq[kPairsInFlight][NCH];
         float gate[kPairsInFlight];
@@ -106,6 +114,22 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
         }
     }
 
+    if (SPLIT) {
+        if (wave > 0) {
+#pragma unroll
+            for (int c = 0; c < NCH; ++c)
+#pragma unroll
+                for (int v = 0; v < V; ++v) partial_rows[(((wave - 1) * NCH + c) * V + v) * kWave + lane] = acc[c][v];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock - 1; ++w)
+#pragma unroll
+            for (int c = 0; c < NCH; ++c)
+#pragma unroll
+                for (int v = 0; v < V; ++v) acc[c][v] += partial_rows[((w * NCH + c) * V + v) * kWave + lane];
+    }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
         const int p = c * kWave + lane;
@@ -120,10 +144,18 @@ int launch_expert_rows(int act, const void* x, const void* down, const void* up,
     const int packets = H / V;
     const int nch = (packets + kWave - 1) / kWave;
     const dim3 block(kWavesPerBlock * kWave);
-    const dim3 grid((unsigned)((T_ + kWavesPerBlock - 1) / kWavesPerBlock));
-#define FMOE_LAUNCH_EXPERT_ACT(N, A)                                                                        \
-    hipLaunchKernelGGL((expert_token_kernel<T, N, A>), grid, block, 0, stream, (const T*)x, (const T*)down, \
-                       (const T*)up, indices, (const T*)gates, (T*)out, T_, H, E, K)
+    // with at most 2048 tokens a workgroup per token still fits the chip at once
+    const bool split = T_ <= 2048 && K > kPairsInFlight;
+    const dim3 grid((unsigned)(split ? T_ : (T_ + kWavesPerBlock - 1) / kWavesPerBlock));
+#define FMOE_LAUNCH_EXPERT_ACT(N, A)                                                                                  \
+    do {                                                                                                              \
+        if (split)                                                                                                    \
+            hipLaunchKernelGGL((expert_token_kernel<T, N, A, true>), grid, block, 0, stream, (const T*)x, (const T*)down, \
+                               (const T*)up, indices, (const T*)gates, (T*)out, T_, H, E, K);                         \
+        else                                                                                                          \
+            hipLaunchKernelGGL((expert_token_kernel<T, N, A, false>), grid, block, 0, stream, (const T*)x, (const T*)down, \
+                               (const T*)up, indices, (const T*)gates, (T*)out, T_, H, E, K);                         \
+    } while (0)
 #define FMOE_LAUNCH_EXPERT(N)                                     \
     do {                                                          \
         if (act == kActSilu) FMOE_LAUNCH_EXPERT_ACT(N, kActSilu); \
