@@ -441,7 +441,7 @@ int launch_expert_slices(int act, const void* x, const void* down, const void* u
 // A 128-byte slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic;
 // up to 8 MiB the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
 // too few pairs to pay for four launches, whole rows are gathered by the one-wave-per-token kernel.
-bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) && T_ * K >= (1ll << 15); }
+bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) && T_ * K >= (1ll << 16); }
 // rows are addressed with 32-bit byte offsets below kBadOffset
 bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
 

@@ -135,7 +135,7 @@ def test_block_c5_shape_fewer_tokens():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("T,H,I,E,K", [(1024, 256, 512, 4096, 32),     # column-slice expert schedule
+@pytest.mark.parametrize("T,H,I,E,K", [(1024, 256, 512, 4096, 64),     # column-slice expert schedule
                                        (96, 128, 256, 1024, 8),        # row-gather expert schedule
                                        (33, 64, 192, 400, 5)])         # ragged: E not a square, odd T and K
 @pytest.mark.parametrize("training", [True, False])

@@ -20,7 +20,7 @@ def pkm_reference(values, w, idx):
 
 
 CASES = [(64, 128, 256, 8),            # row schedule
-         (1024, 256, 4096, 32),        # column-slice schedule (T*K >= 32768, slice fits L2)
+         (1024, 256, 4096, 64),        # column-slice schedule (T*K >= 65536, slice fits L2)
          (33, 1024, 1000, 5),          # ragged
          (16, 2048, 512, 4)]
 
