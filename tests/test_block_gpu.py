@@ -227,3 +227,31 @@ def test_block_of_an_empty_batch():
     m.eval()
     y, logits = m(torch.zeros(2, 0, 128, device="cuda", dtype=torch.bfloat16))
     assert y.shape == (2, 0, 128) and logits.shape == (2, 0, 32)
+
+
+@pytest.mark.parametrize("T", [64, 1024])
+def test_block_forward_under_hip_graph_capture(T):
+    """The single-call forward only launches kernels on the caller's stream (no allocation, no memset, no host
+    synchronisation inside the library), so it can be captured in a HIP graph: every replay equals the eager result."""
+    dtype = torch.bfloat16
+    m, _ = build(256, 512, 4096, 16, True, dtype, seed=4)
+    m.eval()
+    static_x = torch.randn(1, T, 256, generator=torch.Generator().manual_seed(1)).to(dtype).cuda()
+    eager = [m(static_x)[0].clone()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            m(static_x)                                  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y, static_logits = m(static_x)
+    for step in range(3):
+        new_x = torch.randn(1, T, 256, generator=torch.Generator().manual_seed(10 + step)).to(dtype).cuda()
+        expect, expect_logits = m(new_x)                  # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(new_x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, expect) and torch.equal(static_logits, expect_logits), f"replay {step}"
