@@ -183,12 +183,14 @@ int launch_expert_rows(int act, const void* x, const void* down, const void* up,
 //
 // Random 2 KiB row gathers from tables of tens of MiB are served by the Infinity Cache / HBM through the
 // fabric at ~7.6 TB/s on MI355X whatever the kernel does, while gathers from a working set that fits one
-// XCD's 4 MiB L2 run at ~25 TB/s.  So the tables are processed in column slices of 128 bytes (one L2
-// line per row): a slice of a 16384-row table is 2 MiB.  Workgroups are mapped so that XCD x works on
-// slices x, x+8, ... one after the other (workgroup ids are dealt round-robin over the 8 XCDs), each
-// slice streaming through all tokens while its 2 MiB stay resident in that XCD's L2; every table byte
-// leaves HBM / Infinity Cache once.  A wave-wide load fetches the 128-byte pieces of 8 different pairs
-// (8 lanes x 16 bytes each); 8 such loads are in flight per wave.
+// XCD's 4 MiB L2 run at ~25 TB/s.  So the tables are processed in column slices of 256 bytes per row (128 for
+// tables of more than 16384 rows): a slice of a 16384-row table is 4 MiB.  Workgroups are mapped so that XCD x
+// works on slices x, x+8, ... one after the other (workgroup ids are dealt round-robin over the 8 XCDs), each
+// slice streaming through all tokens while it stays resident in that XCD's L2; every table byte leaves HBM /
+// Infinity Cache once.  A wave-wide load fetches the slice's pieces of 4 (or 8) different pairs, 16 bytes per
+// lane; a round of 16 (or 8) such loads, all in flight together, covers 64 pairs.  The wider slice halves the
+// passes over the offsets, coefficients and partial sums: measured 31.9 -> 27.7 us for the scores of 4096
+// tokens x 64 pairs, 117 -> 102 us for 16384 tokens.
 //
 //   prepare : int64 ids -> int32 (-1 if outside [0,E))
 //   scores  : spart[slice][pair] = <x[token, slice cols], down[expert, slice cols]>          (per slice)
@@ -196,9 +198,8 @@ int launch_expert_rows(int act, const void* x, const void* down, const void* up,
 //   states  : out[token, slice cols] = sum_k a[token,k] * up[expert_k, slice cols]           (per slice)
 // `states` needs no cross-slice reduction, so the output is still written exactly once, without atomics.
 // ------------------------------------------------------------------------------------------------
-constexpr int kChunkLanes = 8;     // lanes covering one 128-byte chunk
-constexpr int kChunkPairs = 8;     // pairs per wave-wide load
-constexpr int kSliceLoads = 8;     // wave-wide loads in flight: 64 pairs per round
+// A wave-wide 16-byte load covers 64 / CL rows when CL lanes share one row's chunk (CL = 8: 128-byte slices,
+// CL = 16: 256-byte slices); a round of CL such loads handles 64 pairs.
 constexpr uint32_t kBadOffset = 0xFFF00000u;   // row offset of an invalid id: beyond any table the slice path accepts
 
 // Table rows are addressed through a raw buffer resource: 32-bit byte offsets (no 64-bit address arithmetic
@@ -228,36 +229,42 @@ __device__ inline bool slice_of_block(int num_slices, int blocks_per_slice, int&
     return slice < num_slices;
 }
 
-// p[u] holds, in each of the 8 lanes of a chunk group, that lane's share of pair u's dot product.  Returns in
-// lane c of the group the complete sum of pair u == c: a transposing butterfly (7 cross-lane adds instead of 24).
-__device__ inline float group8_transpose_sum(const float (&p)[8], int c) {
-    const bool b0 = c & 1, b1 = c & 2, b2 = c & 4;
-    float q[4], r[2];
+// p[u] holds, in each of the CL lanes of a chunk group, that lane's share of pair u's dot product.  Returns in
+// lane c of the group the complete sum of pair u == c: a transposing butterfly (CL - 1 cross-lane adds instead of
+// CL * log2(CL)).
+template <int N, int STEP> __device__ inline float xor_step(float v) {
+    if constexpr (STEP == 1) return dpp_move<0xB1>(v);
+    else if constexpr (STEP == 2) return dpp_move<0x4E>(v);
+    else if constexpr (STEP == 8) return dpp_move<0x128>(v);          // rotate the row of 16 by 8
+    else return __shfl_xor(v, STEP, kWave);
+}
+template <int N, int STEP> __device__ inline float transpose_sum(const float (&p)[N], int c) {
+    if constexpr (N == 1) {
+        return p[0];
+    } else {
+        const bool up = c & STEP;
+        float q[N / 2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float keep = b0 ? p[2 * i + 1] : p[2 * i], send = b0 ? p[2 * i] : p[2 * i + 1];
-        q[i] = keep + dpp_move<0xB1>(send);
+        for (int i = 0; i < N / 2; ++i) {
+            const float keep = up ? p[2 * i + 1] : p[2 * i], send = up ? p[2 * i] : p[2 * i + 1];
+            q[i] = keep + xor_step<N, STEP>(send);
+        }
+        return transpose_sum<N / 2, STEP * 2>(q, c);
     }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const float keep = b1 ? q[2 * i + 1] : q[2 * i], send = b1 ? q[2 * i] : q[2 * i + 1];
-        r[i] = keep + dpp_move<0x4E>(send);
-    }
-    const float keep = b2 ? r[1] : r[0], send = b2 ? r[0] : r[1];
-    return keep + __shfl_xor(send, 4, kWave);
 }
 
-template <typename T>
+template <typename T, int CL>
 __global__ __launch_bounds__(256) void expert_scores_slice_kernel(
     const T* __restrict__ x, const T* __restrict__ down, uint32_t table_bytes, const uint32_t* __restrict__ off32,
     float* __restrict__ spart, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
     int tokens_per_block) {
     constexpr int V = Elem<T>::kVec;
+    constexpr int PPL = kWave / CL;                         // pairs per wave-wide load
     int slice, tb;
     if (!slice_of_block(num_slices, blocks_per_slice, slice, tb)) return;
     const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
-    const int c = lane & (kChunkLanes - 1), pg = lane >> 3;
-    const int col = slice * (kChunkLanes * V) + c * V;
+    const int c = lane & (CL - 1), pg = lane / CL;
+    const int col = slice * (CL * V) + c * V;
     const bool col_ok = col < hidden;                       // false only in a partial last slice
     const uint32_t col_bytes = col_ok ? (uint32_t)col * sizeof(T) : 0u;
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
@@ -271,19 +278,19 @@ __global__ __launch_bounds__(256) void expert_scores_slice_kernel(
         const u32x4_t xq = col_ok ? *reinterpret_cast<const u32x4_t*>(x + t * hidden + col) : zero4;
         const uint32_t* tok_off = off32 + t * top_k;
         for (int k0 = 0; k0 < top_k; k0 += kWave) {
-            // one coalesced load brings the row offsets of 64 pairs; lane (pg, c) then needs those of pairs u*8+pg
+            // one coalesced load brings the row offsets of 64 pairs; lane (pg, c) then needs those of pairs u*PPL+pg
             const uint32_t mine = k0 + lane < top_k ? tok_off[k0 + lane] : kBadOffset;
-            u32x4_t w[kSliceLoads];
+            u32x4_t w[CL];
 #pragma unroll
-            for (int u = 0; u < kSliceLoads; ++u) {
-                const uint32_t o = (uint32_t)__builtin_amdgcn_ds_bpermute((u * kChunkPairs + pg) * 4, (int)mine);
+            for (int u = 0; u < CL; ++u) {
+                const uint32_t o = (uint32_t)__builtin_amdgcn_ds_bpermute((u * PPL + pg) * 4, (int)mine);
                 w[u] = load_row_piece(rsrc, o + col_bytes);
             }
-            float part[kSliceLoads];
+            float part[CL];
 #pragma unroll
-            for (int u = 0; u < kSliceLoads; ++u) part[u] = dot16<T>(xq, w[u], 0.0f);
-            const float total = group8_transpose_sum(part, c);     // pair k0 + c*8 + pg
-            const int kk = k0 + c * kChunkPairs + pg;
+            for (int u = 0; u < CL; ++u) part[u] = dot16<T>(xq, w[u], 0.0f);
+            const float total = transpose_sum<CL, 1>(part, c);      // pair k0 + c*PPL + pg
+            const int kk = k0 + c * PPL + pg;
             if (kk < top_k) my_spart[t * top_k + kk] = total;
         }
     }
@@ -320,17 +327,18 @@ template <> __device__ inline void axpy16_pair<bf16_t>(float a0, float a1, u32x4
     }
 }
 
-template <typename T>
+template <typename T, int CL>
 __global__ __launch_bounds__(256) void expert_states_slice_kernel(
     const float* __restrict__ a, const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ off32,
     T* __restrict__ out, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
     int tokens_per_block) {
     constexpr int V = Elem<T>::kVec;
+    constexpr int PPL = kWave / CL;
     int slice, tb;
     if (!slice_of_block(num_slices, blocks_per_slice, slice, tb)) return;
     const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
-    const int c = lane & (kChunkLanes - 1), pg = lane >> 3;
-    const int col = slice * (kChunkLanes * V) + c * V;
+    const int c = lane & (CL - 1), pg = lane / CL;
+    const int col = slice * (CL * V) + c * V;
     const bool col_ok = col < hidden;
     const uint32_t col_bytes = col_ok ? (uint32_t)col * sizeof(T) : 0u;
     const __amdgpu_buffer_rsrc_t rsrc = table_resource(up, table_bytes);
@@ -347,22 +355,22 @@ __global__ __launch_bounds__(256) void expert_states_slice_kernel(
             const bool live = k0 + lane < top_k;
             const uint32_t mine = live ? tok_off[k0 + lane] : kBadOffset;
             const float mine_a = live ? tok_a[k0 + lane] : 0.0f;
-            u32x4_t w[kSliceLoads];
-            float av[kSliceLoads];
+            u32x4_t w[CL];
+            float av[CL];
 #pragma unroll
-            for (int u = 0; u < kSliceLoads; ++u) {
-                const int src = (u * kChunkPairs + pg) * 4;
+            for (int u = 0; u < CL; ++u) {
+                const int src = (u * PPL + pg) * 4;
                 const uint32_t o = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)mine);
                 av[u] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, mine_a)));
                 w[u] = load_row_piece(rsrc, o + col_bytes);      // zeros for an invalid id (out of bounds)
             }
 #pragma unroll
-            for (int u = 0; u < kSliceLoads; u += 2) axpy16_pair<T>(av[u], av[u + 1], w[u], w[u + 1], acc);
+            for (int u = 0; u < CL; u += 2) axpy16_pair<T>(av[u], av[u + 1], w[u], w[u + 1], acc);
         }
-        // sum the 8 pair groups (lanes c, c+8, ..., c+56 hold the same columns)
+        // sum the pair groups (lanes c, c+CL, c+2*CL, ... hold the same columns)
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            acc[v] += dpp_move<0x128>(acc[v]);             // lanes 8 apart
+            if constexpr (CL == 8) acc[v] += dpp_move<0x128>(acc[v]);             // lanes 8 apart
             acc[v] += __shfl_xor(acc[v], 16, kWave);
             acc[v] += __shfl_xor(acc[v], 32, kWave);
         }
@@ -371,14 +379,18 @@ __global__ __launch_bounds__(256) void expert_states_slice_kernel(
 }
 
 struct SlicePlan {
-    int num_slices, blocks_per_slice, tokens_per_block;
+    int chunk_lanes, num_slices, blocks_per_slice, tokens_per_block;
     unsigned grid;
     size_t off_idx32, off_a, off_spart, bytes;
 };
 
-SlicePlan plan_slices(int64_t T_, int H, int K, size_t elt) {
+// A slice is as wide as one XCD's 4 MiB L2 can keep resident: 256 bytes per row up to 16384 rows (fewer passes over
+// the offsets, coefficients and partial sums), 128 bytes beyond.
+SlicePlan plan_slices(int64_t T_, int H, int64_t E, int K, size_t elt) {
     SlicePlan p;
-    p.num_slices = (int)((H * elt + 127) / 128);
+    p.chunk_lanes = E * 256 <= (4ll << 20) ? 16 : 8;
+    const size_t chunk_bytes = (size_t)p.chunk_lanes * 16;
+    p.num_slices = (int)((H * elt + chunk_bytes - 1) / chunk_bytes);
     const int64_t want = (T_ + 3) / 4;                       // at least one token per wave
     p.blocks_per_slice = (int)(want < 1024 ? want : 1024);   // 256 blocks of 4 waves fill one XCD; a few rounds of them
     p.tokens_per_block = (int)((T_ + p.blocks_per_slice - 1) / p.blocks_per_slice);
@@ -395,7 +407,7 @@ SlicePlan plan_slices(int64_t T_, int H, int K, size_t elt) {
 template <typename T>
 int launch_expert_slices_prepared(int act, const void* x, const void* down, const void* up, const void* gates, int64_t T_,
                                   int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
-    const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
+    const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
     char* ws = (char*)workspace;
     const uint32_t* off32 = (const uint32_t*)(ws + p.off_idx32);
     const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
@@ -404,8 +416,14 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
     const int64_t pairs = T_ * K;
     const unsigned flat_grid = (unsigned)((pairs + 255) / 256);
     if (act != kActNone) {
-        hipLaunchKernelGGL((expert_scores_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const T*)x, (const T*)down,
-                           table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+        if (p.chunk_lanes == 16)
+            hipLaunchKernelGGL((expert_scores_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
+                               (const T*)down, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
+                               p.tokens_per_block);
+        else
+            hipLaunchKernelGGL((expert_scores_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
+                               (const T*)down, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
+                               p.tokens_per_block);
         FMOE_CHECK_LAUNCH("fmoe_expert_forward(scores)");
     }
     // without a score (product-key memory) the coefficient is the routing weight: no partial sums are read
@@ -419,9 +437,14 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
         hipLaunchKernelGGL((expert_gate_kernel<T, kActNone>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
                            (const T*)gates, off32, a, pairs, 0);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(gate)");
-    hipLaunchKernelGGL((expert_states_slice_kernel<T>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
-                       (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
-                       p.tokens_per_block);
+    if (p.chunk_lanes == 16)
+        hipLaunchKernelGGL((expert_states_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
+                           (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
+                           p.tokens_per_block);
+    else
+        hipLaunchKernelGGL((expert_states_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
+                           (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
+                           p.tokens_per_block);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(states)");
     return FMOE_OK;
 }
@@ -429,7 +452,7 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
 template <typename T>
 int launch_expert_slices(int act, const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
                          int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
-    const SlicePlan p = plan_slices(T_, H, K, sizeof(T));
+    const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
     uint32_t* off32 = (uint32_t*)((char*)workspace + p.off_idx32);
     const int64_t pairs = T_ * K;
     hipLaunchKernelGGL(expert_prepare_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, indices, off32,
@@ -438,8 +461,8 @@ int launch_expert_slices(int act, const void* x, const void* down, const void* u
     return launch_expert_slices_prepared<T>(act, x, down, up, gates, T_, H, E, K, out, workspace, stream);
 }
 
-// A 128-byte slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic;
-// up to 8 MiB the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
+// A slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic; with 128-byte
+// slices of up to 8 MiB the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
 // too few pairs to pay for four launches, whole rows are gathered by the one-wave-per-token kernel.
 bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) && T_ * K >= (1ll << 16); }
 // rows are addressed with 32-bit byte offsets below kBadOffset
@@ -471,7 +494,7 @@ extern "C" size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidde
     if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0 || top_k <= 0 || !dtype_ok(dtype)) return 0;
     const bool possible = slices_possible(num_experts, hidden, dtype_size(dtype));
     const bool slices = algo == FMOE_EXPERT_SLICES || (algo == FMOE_EXPERT_AUTO && possible && slices_pay(num_tokens, num_experts, top_k));
-    return slices ? plan_slices(num_tokens, hidden, top_k, dtype_size(dtype)).bytes : 0;   // the row schedule needs no scratch
+    return slices ? plan_slices(num_tokens, hidden, num_experts, top_k, dtype_size(dtype)).bytes : 0;   // the row schedule needs no scratch
 }
 
 extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
