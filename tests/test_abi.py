@@ -97,7 +97,9 @@ def test_expert_argument_checks():
     assert isinstance(lib.fmoe_expert_workspace_bytes(1024, 1024, 16384, 64, _C.BF16), int)
     # the size follows the schedule: column slices when a slice of the table fits L2 and there are enough pairs, else none
     sliced = lib.fmoe_expert_workspace_bytes(4096, 1024, 16384, 64, _C.BF16)
-    assert sliced >= 4096 * 64 * (4 + 4 + 16 * 4) and sliced % 256 == 0
+    assert sliced >= 4096 * 64 * (4 + 4 + 8 * 4) and sliced % 256 == 0               # 8 slices of 256 bytes
+    wide = lib.fmoe_expert_workspace_bytes(4096, 1024, 32768, 64, _C.BF16)
+    assert wide >= 4096 * 64 * (4 + 4 + 16 * 4) and wide % 256 == 0                   # 16 slices of 128 bytes
     assert lib.fmoe_expert_workspace_bytes(32768, 2048, 262144, 128, _C.BF16) == 0      # table slice too large for L2
     assert lib.fmoe_expert_workspace_bytes(64, 1024, 16384, 8, _C.BF16) == 0            # too few pairs
     assert lib.fmoe_expert_workspace_bytes_algo(64, 1024, 16384, 8, _C.BF16, _C.EXPERT_SLICES) > 0

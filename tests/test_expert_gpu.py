@@ -31,6 +31,7 @@ def truth64(x, wd, wu, idx, g):
     (37, 72, 50, 5),             # ragged: rows of 9 packets, token count not a multiple of the block
     (3, 8, 4, 1),
     (130, 1000, 300, 70),        # K not a multiple of the 64 pairs a wave handles per round; last slice partial
+    (200, 264, 20000, 40),       # more than 16384 rows: the narrower (128-byte) column slices, last one partial
 ])
 def test_expert_matches_oracle(dtype, T, H, E, K, algo):
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=T + K)
