@@ -202,6 +202,31 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_token_kernel
     }
 }
 
+// Column-slice schedule of the per-token part (same kernels as the forward, fmoe_expert.hip): the partial dot products
+// s = <x, down[e]> and u = <dout, up[e]> come per slice; this kernel sums them and forms every pair's coefficients,
+// gate gradient and histogram entry; dx is then the forward's `states` pass over `down` with coef_down.
+template <typename T>
+__global__ __launch_bounds__(256) void expert_backward_gate_kernel(
+    const float* __restrict__ spart_s, const float* __restrict__ spart_u, const T* __restrict__ gates,
+    const uint32_t* __restrict__ off32, const int64_t* __restrict__ indices, T* __restrict__ dgates,
+    float* __restrict__ coef_up, float* __restrict__ coef_down, int32_t* __restrict__ counts, int64_t pairs, int num_slices) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pairs) return;
+    float s = 0.0f, u = 0.0f;
+    for (int sl = 0; sl < num_slices; ++sl) {
+        s += spart_s[(int64_t)sl * pairs + p];
+        u += spart_u[(int64_t)sl * pairs + p];
+    }
+    const bool valid = off32[p] != kExpertBadOffset;
+    const float gate = Elem<T>::to_f32(gates[p]);
+    const float sig = 1.0f / (1.0f + __expf(-s));
+    const float act = s * sig;
+    coef_up[p] = valid ? act * gate : 0.0f;
+    coef_down[p] = valid ? u * gate * (sig * (1.0f + s * (1.0f - sig))) : 0.0f;
+    dgates[p] = Elem<T>::from_f32(valid ? u * act : 0.0f);
+    if (valid) atomicAdd(&counts[indices[p]], 1);   // integer histogram: the result does not depend on order
+}
+
 __global__ void zero_i32_kernel(int32_t* __restrict__ p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
 }
@@ -358,10 +383,12 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
 }
 
 struct ExpertBwdPlan {
-    size_t off_coef_up, off_coef_down, off_pairs, off_counts, off_cursor, off_offsets, bytes;
+    bool slices;
+    int num_slices;
+    size_t off_coef_up, off_coef_down, off_pairs, off_counts, off_cursor, off_offsets, off_off32, off_spart_s, off_spart_u, bytes;
 };
 
-ExpertBwdPlan plan_expert_backward(int64_t T_, int64_t E, int K) {
+ExpertBwdPlan plan_expert_backward(int64_t T_, int H, int64_t E, int K, int dtype) {
     ExpertBwdPlan p;
     const size_t pairs = (size_t)T_ * K;
     size_t o = 0;
@@ -372,16 +399,24 @@ ExpertBwdPlan plan_expert_backward(int64_t T_, int64_t E, int K) {
     p.off_counts = take((size_t)E * 4);        // counts and cursor are adjacent: one clearing launch
     p.off_cursor = take((size_t)E * 4);
     p.off_offsets = take((size_t)(E + 1) * 4);
+    p.slices = expert_slices_usable(T_, H, E, K, dtype);
+    p.num_slices = p.slices ? expert_slice_count(T_, H, E, K, dtype) : 0;
+    p.off_off32 = p.off_spart_s = p.off_spart_u = o;
+    if (p.slices) {
+        p.off_off32 = take(pairs * 4);
+        p.off_spart_s = take((size_t)p.num_slices * pairs * 4);
+        p.off_spart_u = take((size_t)p.num_slices * pairs * 4);
+    }
     p.bytes = o;
     return p;
 }
 
 template <typename T>
 int launch_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,
-                           const void* gates, int64_t T_, int H, int64_t E, int K, void* dx, void* ddown, void* dup,
+                           const void* gates, int64_t T_, int H, int64_t E, int K, int dtype, void* dx, void* ddown, void* dup,
                            void* dgates, void* workspace, hipStream_t stream) {
     constexpr int V = Elem<T>::kVec;
-    const ExpertBwdPlan p = plan_expert_backward(T_, E, K);
+    const ExpertBwdPlan p = plan_expert_backward(T_, H, E, K, dtype);
     char* ws = (char*)workspace;
     float* coef_up = (float*)(ws + p.off_coef_up);
     float* coef_down = (float*)(ws + p.off_coef_down);
@@ -398,16 +433,30 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
     const int64_t clear = (int64_t)((p.off_cursor - p.off_counts) / 4) + E;
     hipLaunchKernelGGL(zero_i32_kernel, dim3(256), dim3(256), 0, stream, counts, clear);
     FMOE_CHECK_LAUNCH("fmoe_expert_backward(clear)");
+    if (p.slices) {
+        uint32_t* off32 = (uint32_t*)(ws + p.off_off32);
+        float* spart_s = (float*)(ws + p.off_spart_s);
+        float* spart_u = (float*)(ws + p.off_spart_u);
+        if (int rc = expert_slice_prepare(indices, off32, pairs, H, E, dtype, stream)) return rc;
+        if (int rc = expert_slice_scores(x, down, off32, spart_s, T_, H, E, K, dtype, stream)) return rc;
+        if (int rc = expert_slice_scores(dout, up, off32, spart_u, T_, H, E, K, dtype, stream)) return rc;
+        hipLaunchKernelGGL((expert_backward_gate_kernel<T>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream,
+                           (const float*)spart_s, (const float*)spart_u, (const T*)gates, (const uint32_t*)off32, indices,
+                           (T*)dgates, coef_up, coef_down, counts, pairs, p.num_slices);
+        FMOE_CHECK_LAUNCH("fmoe_expert_backward(coefficients)");
+        if (int rc = expert_slice_states(coef_down, down, off32, dx, T_, H, E, K, dtype, stream)) return rc;
+    } else {
 #define FMOE_LAUNCH_TOKEN(N)                                                                                          \
-    hipLaunchKernelGGL((expert_backward_token_kernel<T, N>), token_grid, block, 0, stream, (const T*)dout, (const T*)x, \
-                       (const T*)down, (const T*)up, indices, (const T*)gates, (T*)dx, (T*)dgates, coef_up, coef_down,  \
-                       counts, T_, H, E, K)
-    if (nch <= 1) FMOE_LAUNCH_TOKEN(1);
-    else if (nch <= 2) FMOE_LAUNCH_TOKEN(2);
-    else if (nch <= 4) FMOE_LAUNCH_TOKEN(4);
-    else FMOE_LAUNCH_TOKEN(8);
+        hipLaunchKernelGGL((expert_backward_token_kernel<T, N>), token_grid, block, 0, stream, (const T*)dout, (const T*)x, \
+                           (const T*)down, (const T*)up, indices, (const T*)gates, (T*)dx, (T*)dgates, coef_up, coef_down,  \
+                           counts, T_, H, E, K)
+        if (nch <= 1) FMOE_LAUNCH_TOKEN(1);
+        else if (nch <= 2) FMOE_LAUNCH_TOKEN(2);
+        else if (nch <= 4) FMOE_LAUNCH_TOKEN(4);
+        else FMOE_LAUNCH_TOKEN(8);
 #undef FMOE_LAUNCH_TOKEN
-    FMOE_CHECK_LAUNCH("fmoe_expert_backward(tokens)");
+        FMOE_CHECK_LAUNCH("fmoe_expert_backward(tokens)");
+    }
 
     hipLaunchKernelGGL(expert_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, (const int32_t*)counts, offsets, E);
     FMOE_CHECK_LAUNCH("fmoe_expert_backward(scan)");
@@ -498,7 +547,7 @@ extern "C" int fmoe_swiglu_backward(const void* dc, const void* a, const void* b
 
 extern "C" size_t fmoe_expert_backward_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
     if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0 || top_k <= 0 || !fmoe::dtype_ok(dtype)) return 0;
-    return fmoe::plan_expert_backward(num_tokens, num_experts, top_k).bytes;
+    return fmoe::plan_expert_backward(num_tokens, hidden, num_experts, top_k, dtype).bytes;
 }
 
 extern "C" int fmoe_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,
@@ -531,12 +580,12 @@ extern "C" int fmoe_expert_backward(const void* dout, const void* x, const void*
         return FMOE_OK;
     }
     FMOE_REQUIRE(indices && gates && dgates, FMOE_ERR_NULL_POINTER, "fmoe_expert_backward: null indices/gates with top_k=%d", top_k);
-    const size_t need = plan_expert_backward(num_tokens, num_experts, top_k).bytes;
+    const size_t need = plan_expert_backward(num_tokens, hidden, num_experts, top_k, dtype).bytes;
     FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
                  "fmoe_expert_backward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     switch (dtype) {
-        case FMOE_F32: return launch_expert_backward<float>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dx, ddown, dup, dgates, workspace, s);
-        case FMOE_BF16: return launch_expert_backward<bf16_t>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dx, ddown, dup, dgates, workspace, s);
-        default: return launch_expert_backward<f16_t>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dx, ddown, dup, dgates, workspace, s);
+        case FMOE_F32: return launch_expert_backward<float>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dtype, dx, ddown, dup, dgates, workspace, s);
+        case FMOE_BF16: return launch_expert_backward<bf16_t>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dtype, dx, ddown, dup, dgates, workspace, s);
+        default: return launch_expert_backward<f16_t>(dout, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, dtype, dx, ddown, dup, dgates, workspace, s);
     }
 }

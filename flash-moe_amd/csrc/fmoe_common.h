@@ -56,6 +56,17 @@ uint32_t* expert_workspace_offsets(void* workspace);
 int expert_slices_prepared(const void* x, const void* down, const void* up, const void* gates, int64_t num_tokens,
                            int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
                            hipStream_t stream);
+// The same schedule stage by stage (for the backward pass): row byte offsets of the ids (kExpertBadOffset for an id
+// outside [0,E)), per-slice partial dot products spart[slice][pair] = <x[token, slice], table[expert, slice]>, and
+// out[token, :] = sum_k coef[token,k] * table[expert_k, :].  expert_slice_count is the number of slices.
+constexpr uint32_t kExpertBadOffset = 0xFFF00000u;   // beyond any table the slice schedule accepts
+int expert_slice_count(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
+int expert_slice_prepare(const int64_t* indices, uint32_t* off32, int64_t pairs, int hidden, int64_t num_experts, int dtype,
+                         hipStream_t stream);
+int expert_slice_scores(const void* x, const void* table, const uint32_t* off32, float* spart, int64_t num_tokens, int hidden,
+                        int64_t num_experts, int top_k, int dtype, hipStream_t stream);
+int expert_slice_states(const float* coef, const void* table, const uint32_t* off32, void* out, int64_t num_tokens, int hidden,
+                        int64_t num_experts, int top_k, int dtype, hipStream_t stream);
 
 // Plain library GEMM (rocBLAS, loaded on first use) for the operand layouts of the backward passes; row-major
 // C[M,N] = A[M,K] B[K,N] (kBlasNN) or A[K,M]^T B[K,N] (kBlasTN), C = product + beta * C.  Defined in fmoe_mlp_backward.hip.

@@ -200,7 +200,7 @@ int launch_expert_rows(int act, const void* x, const void* down, const void* up,
 // ------------------------------------------------------------------------------------------------
 // A wave-wide 16-byte load covers 64 / CL rows when CL lanes share one row's chunk (CL = 8: 128-byte slices,
 // CL = 16: 256-byte slices); a round of CL such loads handles 64 pairs.
-constexpr uint32_t kBadOffset = 0xFFF00000u;   // row offset of an invalid id: beyond any table the slice path accepts
+constexpr uint32_t kBadOffset = kExpertBadOffset;
 
 // Table rows are addressed through a raw buffer resource: 32-bit byte offsets (no 64-bit address arithmetic
 // per load) and hardware bounds checking, so the row of an invalid id reads as zeros.
@@ -403,6 +403,38 @@ SlicePlan plan_slices(int64_t T_, int H, int64_t E, int K, size_t elt) {
     return p;
 }
 
+template <typename T>
+int launch_slice_scores(const void* x, const void* table, const uint32_t* off32, float* spart, int64_t T_, int H, int64_t E,
+                        int K, hipStream_t stream) {
+    const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
+    const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
+    if (p.chunk_lanes == 16)
+        hipLaunchKernelGGL((expert_scores_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
+                           (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
+                           p.tokens_per_block);
+    else
+        hipLaunchKernelGGL((expert_scores_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
+                           (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
+                           p.tokens_per_block);
+    FMOE_CHECK_LAUNCH("routed experts (slice scores)");
+    return FMOE_OK;
+}
+
+template <typename T>
+int launch_slice_states(const float* a, const void* table, const uint32_t* off32, void* out, int64_t T_, int H, int64_t E,
+                        int K, hipStream_t stream) {
+    const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
+    const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
+    if (p.chunk_lanes == 16)
+        hipLaunchKernelGGL((expert_states_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, a, (const T*)table,
+                           table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+    else
+        hipLaunchKernelGGL((expert_states_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, a, (const T*)table,
+                           table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+    FMOE_CHECK_LAUNCH("routed experts (slice states)");
+    return FMOE_OK;
+}
+
 // Scores, gate and states launches on row offsets that already sit at the start of the workspace.
 template <typename T>
 int launch_expert_slices_prepared(int act, const void* x, const void* down, const void* up, const void* gates, int64_t T_,
@@ -410,22 +442,12 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
     const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
     char* ws = (char*)workspace;
     const uint32_t* off32 = (const uint32_t*)(ws + p.off_idx32);
-    const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
     float* a = (float*)(ws + p.off_a);
     float* spart = (float*)(ws + p.off_spart);
     const int64_t pairs = T_ * K;
     const unsigned flat_grid = (unsigned)((pairs + 255) / 256);
-    if (act != kActNone) {
-        if (p.chunk_lanes == 16)
-            hipLaunchKernelGGL((expert_scores_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
-                               (const T*)down, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
-                               p.tokens_per_block);
-        else
-            hipLaunchKernelGGL((expert_scores_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
-                               (const T*)down, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
-                               p.tokens_per_block);
-        FMOE_CHECK_LAUNCH("fmoe_expert_forward(scores)");
-    }
+    if (act != kActNone)
+        if (int rc = launch_slice_scores<T>(x, down, off32, spart, T_, H, E, K, stream)) return rc;
     // without a score (product-key memory) the coefficient is the routing weight: no partial sums are read
     if (act == kActSilu)
         hipLaunchKernelGGL((expert_gate_kernel<T, kActSilu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
@@ -437,16 +459,7 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
         hipLaunchKernelGGL((expert_gate_kernel<T, kActNone>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
                            (const T*)gates, off32, a, pairs, 0);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(gate)");
-    if (p.chunk_lanes == 16)
-        hipLaunchKernelGGL((expert_states_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
-                           (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
-                           p.tokens_per_block);
-    else
-        hipLaunchKernelGGL((expert_states_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const float*)a,
-                           (const T*)up, table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice,
-                           p.tokens_per_block);
-    FMOE_CHECK_LAUNCH("fmoe_expert_forward(states)");
-    return FMOE_OK;
+    return launch_slice_states<T>(a, up, off32, out, T_, H, E, K, stream);
 }
 
 template <typename T>
@@ -483,6 +496,37 @@ int expert_slices_prepared(const void* x, const void* down, const void* up, cons
         case FMOE_F32: return launch_expert_slices_prepared<float>(kActSilu, x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
         case FMOE_BF16: return launch_expert_slices_prepared<bf16_t>(kActSilu, x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
         default: return launch_expert_slices_prepared<f16_t>(kActSilu, x, down, up, gates, num_tokens, hidden, num_experts, top_k, out, workspace, stream);
+    }
+}
+
+// The stages of the column-slice schedule one by one, for the backward pass (fmoe_backward.hip).
+int expert_slice_count(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
+    return plan_slices(num_tokens, hidden, num_experts, top_k, dtype_size(dtype)).num_slices;
+}
+
+int expert_slice_prepare(const int64_t* indices, uint32_t* off32, int64_t pairs, int hidden, int64_t num_experts, int dtype,
+                         hipStream_t stream) {
+    hipLaunchKernelGGL(expert_prepare_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, indices, off32,
+                       pairs, num_experts, (uint32_t)(hidden * dtype_size(dtype)));
+    FMOE_CHECK_LAUNCH("routed experts (slice offsets)");
+    return FMOE_OK;
+}
+
+int expert_slice_scores(const void* x, const void* table, const uint32_t* off32, float* spart, int64_t num_tokens, int hidden,
+                        int64_t num_experts, int top_k, int dtype, hipStream_t stream) {
+    switch (dtype) {
+        case FMOE_F32: return launch_slice_scores<float>(x, table, off32, spart, num_tokens, hidden, num_experts, top_k, stream);
+        case FMOE_BF16: return launch_slice_scores<bf16_t>(x, table, off32, spart, num_tokens, hidden, num_experts, top_k, stream);
+        default: return launch_slice_scores<f16_t>(x, table, off32, spart, num_tokens, hidden, num_experts, top_k, stream);
+    }
+}
+
+int expert_slice_states(const float* coef, const void* table, const uint32_t* off32, void* out, int64_t num_tokens, int hidden,
+                        int64_t num_experts, int top_k, int dtype, hipStream_t stream) {
+    switch (dtype) {
+        case FMOE_F32: return launch_slice_states<float>(coef, table, off32, out, num_tokens, hidden, num_experts, top_k, stream);
+        case FMOE_BF16: return launch_slice_states<bf16_t>(coef, table, off32, out, num_tokens, hidden, num_experts, top_k, stream);
+        default: return launch_slice_states<f16_t>(coef, table, off32, out, num_tokens, hidden, num_experts, top_k, stream);
     }
 }
 
