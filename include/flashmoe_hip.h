@@ -119,7 +119,8 @@ int fmoe_expert_forward(const void* x, const void* down, const void* up, const i
 
 /* Same operation with the schedule chosen by the caller instead of by problem size (fmoe_expert_forward
  * passes FMOE_EXPERT_AUTO).  Both schedules compute the formula above; they differ in how the table rows
- * travel: whole rows per (token, expert) pair, or 128-byte column slices kept resident in each XCD's L2.
+ * travel: whole rows per (token, expert) pair, or 128- or 256-byte column slices, each worked through by
+ * one XCD (one L2) at a time.
  * The reference has one schedule (expert-centric Triton kernels, flash_expert.py:580-651). */
 typedef enum {
     FMOE_EXPERT_AUTO = 0,
