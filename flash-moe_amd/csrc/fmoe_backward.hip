@@ -1,6 +1,7 @@
 // Backward passes of the router op, the SwiGLU gate and the routed-expert op for gfx950.
 //
 //   router  : drouter_logits[0,t,i] = sum_{k : idx[t,k] / nk == i} dscores[t,k],  [1,t,j] likewise with idx % nk
+//   route   : gates = exp(top-k sums of the per-half log-softmax), renormalised or not -> gradient of the gate logits
 //   swiglu  : c = silu(a) * b  ->  da = dc * (silu(a) * (1 - sigmoid(a)) + sigmoid(a)) * b,  db = dc * silu(a)
 //   experts : out[t] = sum_k silu(s) * g * up[e],  s = <x[t], down[e]>,  e = idx[t,k]:
 //               da_p   = <dout[t], up[e]>                 dg_p = da_p * silu(s)
@@ -66,6 +67,97 @@ int launch_router_backward(const void* dscores, const int64_t* indices, void* dl
     hipLaunchKernelGGL((router_backward_kernel<T>), dim3(grid), dim3(kBwdWaves * kWave), waves * per_wave, stream,
                        (const T*)dscores, indices, (T*)dlogits, T_, nk, K, waves);
     FMOE_CHECK_LAUNCH("fmoe_router_topk_backward");
+    return FMOE_OK;
+}
+
+// Routing stage between the gate logits and the gates, backward in one launch: exp / renormalisation, the scatter of the
+// score gradients onto the two key rows, and the per-half log-softmax.  One wave per token; the log-probabilities are
+// recomputed from the fp32 logits exactly as the forward computes them ((v - max) - log(sum exp(v - max))).
+//   s_k = lp0[i_k] + lp1[j_k],  e_k = exp(s_k),  g_k = e_k  or  e_k / sum_m e_m
+//   ds_k = dg_k * e_k                       (no renormalisation)
+//   ds_k = g_k * (dg_k - sum_m dg_m g_m)    (renormalised)
+//   dlp[h][i] = sum of ds_k over the pairs that use key i of half h
+//   dlogits[h][i] = dlp[h][i] - softmax(logits[h])[i] * sum_i dlp[h][i]   (+ the gradient of the returned logits)
+template <typename T>
+__global__ __launch_bounds__(kBwdWaves* kWave) void route_backward_kernel(
+    const T* __restrict__ dgates, const int64_t* __restrict__ indices, const float* __restrict__ logits,
+    const T* __restrict__ dlogits_extra, float* __restrict__ dlogits, int64_t num_tokens, int nk, int top_k,
+    int norm_topk_prob, int waves_per_block) {
+    extern __shared__ float acc_all[];   // [waves_per_block][2 * nk], one private row pair per wave
+    const int lane = lane_id();
+    const int wave = (int)(threadIdx.x >> 6);
+    const int64_t token = (int64_t)blockIdx.x * waves_per_block + wave;
+    if (wave >= waves_per_block || token >= num_tokens) return;   // whole waves leave; nobody waits on them
+    float* acc = acc_all + (size_t)wave * 2 * nk;
+    const float* row = logits + token * 2 * nk;
+    float shift[2], lse[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        float mx = -INFINITY;
+        for (int p = lane; p < nk; p += kWave) mx = fmaxf(mx, row[h * nk + p]);
+        mx = wave_max(mx);
+        float se = 0.0f;
+        for (int p = lane; p < nk; p += kWave) se += expf(row[h * nk + p] - mx);
+        shift[h] = mx;
+        lse[h] = logf(wave_sum(se));
+    }
+    for (int p = lane; p < 2 * nk; p += kWave) acc[p] = 0.0f;
+    __builtin_amdgcn_wave_barrier();
+    const int64_t num_pairs = (int64_t)nk * nk;
+    // first pass (renormalised gates only): sum_m e_m and sum_m dg_m e_m
+    float total = 1.0f, dot = 0.0f;
+    if (norm_topk_prob) {
+        float te = 0.0f, td = 0.0f;
+        for (int k = lane; k < top_k; k += kWave) {
+            const int64_t id = indices[token * top_k + k];
+            if (id >= 0 && id < num_pairs) {
+                const int i = (int)(id / nk), j = (int)(id % nk);
+                const float e = expf(((row[i] - shift[0]) - lse[0]) + ((row[nk + j] - shift[1]) - lse[1]));
+                te += e;
+                td = __builtin_fmaf(Elem<T>::to_f32(dgates[token * top_k + k]), e, td);
+            }
+        }
+        total = wave_sum(te);
+        dot = wave_sum(td) / total;          // sum_m dg_m g_m
+    }
+    // LDS adds of one instruction that hit the same address are applied one after the other by the LDS unit, and the
+    // instructions of a wave execute in order, so the sum has a fixed order for given inputs
+    for (int k = lane; k < top_k; k += kWave) {
+        const int64_t id = indices[token * top_k + k];
+        if (id >= 0 && id < num_pairs) {
+            const int i = (int)(id / nk), j = (int)(id % nk);
+            const float e = expf(((row[i] - shift[0]) - lse[0]) + ((row[nk + j] - shift[1]) - lse[1]));
+            const float dg = Elem<T>::to_f32(dgates[token * top_k + k]);
+            const float ds = norm_topk_prob ? (e / total) * (dg - dot) : dg * e;
+            __hip_atomic_fetch_add(&acc[i], ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            __hip_atomic_fetch_add(&acc[nk + j], ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        float sum = 0.0f;
+        for (int p = lane; p < nk; p += kWave) sum += acc[h * nk + p];
+        sum = wave_sum(sum);
+        for (int p = lane; p < nk; p += kWave) {
+            const int64_t at = token * 2 * nk + h * nk + p;
+            float d = acc[h * nk + p] - expf((row[h * nk + p] - shift[h]) - lse[h]) * sum;
+            if (dlogits_extra != nullptr) d += Elem<T>::to_f32(dlogits_extra[at]);
+            dlogits[at] = d;
+        }
+    }
+}
+
+template <typename T>
+int launch_route_backward(const void* dgates, const int64_t* indices, const float* logits, const void* dlogits_extra,
+                          float* dlogits, int64_t T_, int nk, int K, int norm, hipStream_t stream) {
+    const size_t per_wave = (size_t)2 * nk * sizeof(float);
+    int waves = (int)((48 * 1024) / per_wave);
+    waves = waves < 1 ? 1 : (waves > kBwdWaves ? kBwdWaves : waves);
+    const unsigned grid = (unsigned)((T_ + waves - 1) / waves);
+    hipLaunchKernelGGL((route_backward_kernel<T>), dim3(grid), dim3(kBwdWaves * kWave), waves * per_wave, stream,
+                       (const T*)dgates, indices, logits, (const T*)dlogits_extra, dlogits, T_, nk, K, norm, waves);
+    FMOE_CHECK_LAUNCH("fmoe_route_backward");
     return FMOE_OK;
 }
 
@@ -528,6 +620,26 @@ extern "C" int fmoe_router_topk_backward(const void* dscores, const int64_t* ind
         case FMOE_F32: return launch_router_backward<float>(dscores, indices, drouter_logits, num_tokens, num_keys, top_k, s);
         case FMOE_BF16: return launch_router_backward<bf16_t>(dscores, indices, drouter_logits, num_tokens, num_keys, top_k, s);
         default: return launch_router_backward<f16_t>(dscores, indices, drouter_logits, num_tokens, num_keys, top_k, s);
+    }
+}
+
+extern "C" int fmoe_route_backward(const void* dgates, const int64_t* indices, const float* logits_fp32, const void* dlogits_extra,
+                                   int64_t num_tokens, int num_keys, int top_k, int dtype, int norm_topk_prob,
+                                   float* dlogits_fp32, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_route_backward: unknown dtype %d", dtype);
+    FMOE_REQUIRE(num_tokens >= 0 && num_keys > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
+                 "fmoe_route_backward: bad shape T=%lld nk=%d K=%d", (long long)num_tokens, num_keys, top_k);
+    FMOE_REQUIRE(num_keys <= 8192, FMOE_ERR_UNSUPPORTED, "fmoe_route_backward: num_keys=%d > 8192", num_keys);
+    if (num_tokens == 0) return FMOE_OK;
+    FMOE_REQUIRE(logits_fp32 && dlogits_fp32 && (top_k == 0 || (dgates && indices)), FMOE_ERR_NULL_POINTER,
+                 "fmoe_route_backward: null tensor pointer");
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case FMOE_F32: return launch_route_backward<float>(dgates, indices, logits_fp32, dlogits_extra, dlogits_fp32, num_tokens, num_keys, top_k, norm_topk_prob, s);
+        case FMOE_BF16: return launch_route_backward<bf16_t>(dgates, indices, logits_fp32, dlogits_extra, dlogits_fp32, num_tokens, num_keys, top_k, norm_topk_prob, s);
+        default: return launch_route_backward<f16_t>(dgates, indices, logits_fp32, dlogits_extra, dlogits_fp32, num_tokens, num_keys, top_k, norm_topk_prob, s);
     }
 }
 

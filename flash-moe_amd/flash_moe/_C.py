@@ -48,6 +48,7 @@ SIGNATURES = {
     "fmoe_peer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_pkm_forward": (_int, [_vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_router_topk_backward": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
+    "fmoe_route_backward": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _vp, _vp]),
     "fmoe_router_workspace_stats_offset": (_sz, [_i64, _int, _int]),
     "fmoe_router_prologue_backward_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
     "fmoe_router_prologue_backward": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _int, _int, _int, _vp, _vp, _vp, _sz, _vp]),

@@ -11,8 +11,10 @@ pair (:55-105).
   shared SwiGLU MLP + add                                           ``fmoe_mlp_forward`` (the add is the second
                                                                     GEMM's epilogue)
 ``forward_staged`` runs the same three stages as three calls.  When gradients are being recorded ``forward`` takes
-``forward_autograd`` instead: the reference's own composition (batch norm + router gate, log-softmax, then the router,
-expert and MLP ops, flash_moe/modules/flash_moe.py:62-101); every stage but the log-softmax carries a HIP backward pass.
+``forward_autograd`` instead: one autograd node whose forward is those three calls (keeping what the backward needs)
+and whose backward is the library's backward calls.  ``forward_autograd_ops`` is the reference's own composition
+(batch norm + router gate, log-softmax, then the router, expert and MLP ops, flash_moe/modules/flash_moe.py:62-101) on the
+differentiable per-op functions; both give the same gradients.
 
 Routing is evaluated in fp32 whatever the module dtype: the normalised activations are rounded to the
 module dtype exactly as the reference does, but their product with the router gate, the log-softmax
@@ -29,7 +31,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from flash_moe.ops.hip.flash_block import block_forward
+from flash_moe.ops.hip.flash_block import block_forward, block_forward_autograd
 from flash_moe.ops.hip.flash_expert import expert_forward, flash_expert_func
 from flash_moe.ops.hip.flash_mlp import flash_mlp_func, mlp_forward
 from flash_moe.ops.hip.flash_router import flash_router_func, router_forward, router_prologue
@@ -100,8 +102,24 @@ class FlashMoE(nn.Module):
         return out.view(bsz, seq_len, self.hidden_size), router_logits
 
     def forward_autograd(self, hidden_states: torch.Tensor):
-        """Differentiable forward.  Routing is evaluated in fp32 as on the fused path: the normalised activations are
-        rounded to the module dtype, their product with the router gate and the log-softmax are fp32."""
+        """Differentiable forward: one autograd node around the library's forward and backward calls."""
+        bsz, seq_len, _ = hidden_states.shape
+        tokens = hidden_states.reshape(bsz * seq_len, self.hidden_size)
+        num_tokens = tokens.shape[0]
+        if num_tokens == 0 or self.top_k == 0:
+            return self.forward_autograd_ops(hidden_states)
+        out, logits = block_forward_autograd(
+            tokens, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, self.router_gate.weight,
+            self.router_norm, self.down_embed.weight, self.up_embed.weight, self.num_keys, self.top_k, self.norm_topk_prob,
+        )
+        router_logits = logits.view(num_tokens, 2, self.num_keys).transpose(0, 1)
+        return out.view(bsz, seq_len, self.hidden_size), router_logits
+
+    def forward_autograd_ops(self, hidden_states: torch.Tensor):
+        """Differentiable forward op by op, as the reference composes it (flash_moe/modules/flash_moe.py:62-101): the
+        differentiable router prologue, torch's log-softmax, then the router, expert and MLP functions.  Routing is
+        evaluated in fp32 as on the fused path: the normalised activations are rounded to the module dtype, their product
+        with the router gate and the log-softmax are fp32."""
         bsz, seq_len, _ = hidden_states.shape
         tokens = hidden_states.reshape(bsz * seq_len, self.hidden_size)
         num_tokens = tokens.shape[0]

@@ -55,3 +55,56 @@ def block_forward(tokens: torch.Tensor, gate_proj: torch.Tensor, up_proj: torch.
     if return_routing:
         return out, logits, indices, gates
     return out, logits
+
+
+class FlashMoEBlockFunc(torch.autograd.Function):
+    """The block with gradients for the tokens and every weight, library calls only.
+
+    Forward: the three calls the single-call forward is made of (``fmoe_router_forward``, ``fmoe_expert_forward``,
+    ``fmoe_mlp_gate_up_save`` + ``fmoe_mlp_down`` with the experts' output as residual), keeping what the backward needs:
+    ids, gates, the fp32 gate logits, the batch-norm statistics and the MLP's gate / up products.  Backward:
+    ``fmoe_mlp_backward``, ``fmoe_expert_backward``, ``fmoe_route_backward``, ``fmoe_router_prologue_backward`` and the
+    sum of the three token gradients.  The reference reaches the same gradients through autograd of its eager ops
+    around the three Triton functions (flash_moe/modules/flash_moe.py:55-105)."""
+
+    @staticmethod
+    def forward(ctx, tokens, gate_proj, up_proj, down_proj, router_gate, down_embed, up_embed, norm, num_expert_keys,
+                num_experts_per_tok, norm_topk_prob):
+        from flash_moe.ops.hip.flash_expert import expert_forward
+        from flash_moe.ops.hip.flash_mlp import mlp_forward_saving
+        from flash_moe.ops.hip.flash_router import router_forward
+
+        x = tokens.contiguous()
+        training = bool(norm.training)
+        logits, _, indices, gates, logits32, stats = router_forward(
+            x, router_gate, norm, num_expert_keys, num_experts_per_tok, norm_topk_prob, return_logits32=True, return_stats=True)
+        experts = expert_forward(x, down_embed, up_embed, indices, gates)
+        out, saved = mlp_forward_saving(x, gate_proj, up_proj, down_proj, residual=experts)
+        ctx.save_for_backward(x, gate_proj, up_proj, down_proj, router_gate, down_embed, up_embed, indices, gates, logits32,
+                              stats, saved)
+        ctx.training, ctx.num_expert_keys, ctx.norm_topk_prob = training, num_expert_keys, bool(norm_topk_prob)
+        return out, logits
+
+    @staticmethod
+    def backward(ctx, dout, dlogits):
+        from flash_moe.ops.hip.flash_expert import expert_backward
+        from flash_moe.ops.hip.flash_mlp import mlp_backward
+        from flash_moe.ops.hip.flash_router import route_backward, router_prologue_backward
+
+        x, wg, wu, wd, wr, ed, eu, indices, gates, logits32, stats, saved = ctx.saved_tensors
+        if dout is None:
+            dout = torch.zeros_like(x)
+        dout = dout.contiguous()
+        dx, dwg, dwu, dwd = mlp_backward(dout, x, wg, wu, wd, saved)
+        dx_experts, ded, deu, dgates = expert_backward(dout, x, ed, eu, indices, gates)
+        dlogits32 = route_backward(dgates, indices, logits32, ctx.num_expert_keys, ctx.norm_topk_prob, dlogits)
+        dx_router, dwr = router_prologue_backward(dlogits32, x, wr, stats, ctx.training)
+        dx.add_(dx_experts).add_(dx_router)
+        return dx, dwg, dwu, dwd, dwr, ded, deu, None, None, None, None
+
+
+def block_forward_autograd(tokens, gate_proj, up_proj, down_proj, router_gate, norm, down_embed, up_embed, num_expert_keys,
+                           num_experts_per_tok, norm_topk_prob=False):
+    """Differentiable ``block_forward``: ``(out [T, H], router_logits [T, 2*nk])``."""
+    return FlashMoEBlockFunc.apply(tokens, gate_proj, up_proj, down_proj, router_gate, down_embed, up_embed, norm,
+                                   num_expert_keys, num_experts_per_tok, norm_topk_prob)

@@ -48,7 +48,7 @@ def mlp_forward(x, gate_weight, up_weight, down_weight, residual: Optional[torch
     return out.view(x.shape)
 
 
-def mlp_forward_saving(x, gate_weight, up_weight, down_weight):
+def mlp_forward_saving(x, gate_weight, up_weight, down_weight, residual: Optional[torch.Tensor] = None):
     """``mlp_forward`` that also returns the [2, T, I] gate and up products for ``mlp_backward`` (``fmoe_mlp_gate_up_save``
     then ``fmoe_mlp_down``), as the reference's SwiGLU function saves them (flash_moe/ops/triton/flash_mlp.py:153-159)."""
     hidden, inter = x.shape[-1], gate_weight.shape[0]
@@ -56,8 +56,13 @@ def mlp_forward_saving(x, gate_weight, up_weight, down_weight):
         raise ValueError("expected gate_weight/up_weight (intermediate, hidden) and down_weight (hidden, intermediate)")
     if any(t.dtype != x.dtype for t in (gate_weight, up_weight, down_weight)):
         raise TypeError(f"all weights must have the dtype of x ({x.dtype})")
-    dev = _C.require_gpu(x, gate_weight, up_weight, down_weight)
+    dev = _C.require_gpu(x, gate_weight, up_weight, down_weight, residual)
     x2 = x.contiguous().view(-1, hidden)
+    res = None
+    if residual is not None:
+        if residual.shape != x.shape or residual.dtype != x.dtype:
+            raise ValueError("residual must have the shape and dtype of x")
+        res = residual.contiguous().view(-1, hidden)
     wg, wu, wd = gate_weight.contiguous(), up_weight.contiguous(), down_weight.contiguous()
     num_tokens, code = x2.shape[0], _C.dtype_code(x.dtype)
     act = torch.empty((num_tokens, inter), device=dev, dtype=x.dtype)
@@ -68,7 +73,7 @@ def mlp_forward_saving(x, gate_weight, up_weight, down_weight):
         stream = _C.current_stream(dev)
         _C.check(L.fmoe_mlp_gate_up_save(_C.ptr(x2), _C.ptr(wg), _C.ptr(wu), num_tokens, hidden, inter, code, _C.ptr(act),
                                          _C.ptr(saved), stream), "flash_mlp")
-        _C.check(L.fmoe_mlp_down(_C.ptr(act), _C.ptr(wd), num_tokens, hidden, inter, code, None, _C.ptr(out), stream), "flash_mlp")
+        _C.check(L.fmoe_mlp_down(_C.ptr(act), _C.ptr(wd), num_tokens, hidden, inter, code, _C.ptr(res), _C.ptr(out), stream), "flash_mlp")
     return out.view(x.shape), saved
 
 

@@ -75,13 +75,15 @@ def check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_pe
 
 
 def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.nn.BatchNorm1d, num_expert_keys: int,
-                   num_experts_per_tok: int, norm_topk_prob: bool = False, return_logits32: bool = False):
+                   num_experts_per_tok: int, norm_topk_prob: bool = False, return_logits32: bool = False,
+                   return_stats: bool = False):
     """The block's whole routing stage in one call of ``fmoe_router_forward``: batch-norm (training or evaluation
     mode, taken from ``norm.training``; its running statistics are updated in place), the router gate, the per-half
     log-softmax, the product-key top-k and the gates (flash_moe/modules/flash_moe.py:62-85).
 
     Returns ``(router_logits [T, 2*nk] in tokens.dtype, scores [T,K] fp32, indices [T,K] int64, gates [T,K] in
-    tokens.dtype)``, plus the fp32 logits the routing was computed from when ``return_logits32`` is set.
+    tokens.dtype)``, plus the fp32 logits the routing was computed from when ``return_logits32`` is set, plus the
+    batch-norm mean and 1/sqrt(var + eps) used ([2*H] fp32, a view of the call's workspace) when ``return_stats`` is set.
     """
     dev, training = check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok)
     T, H = tokens.shape
@@ -104,9 +106,13 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
             _C.ptr(ws), ws_bytes, _C.current_stream(dev),
         )
     _C.check(status, "flash_router")
+    result = (logits, scores, indices, gates)
     if return_logits32:
-        return logits, scores, indices, gates, logits32
-    return logits, scores, indices, gates
+        result += (logits32,)
+    if return_stats:
+        off = L.fmoe_router_workspace_stats_offset(T, H, num_expert_keys)
+        result += (ws[off:off + 2 * H * 4].view(torch.float32),)
+    return result
 
 
 class RouterPrologueFunc(torch.autograd.Function):
@@ -144,26 +150,63 @@ class RouterPrologueFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dlogits32, dlogits):
         x, w, stats = ctx.saved_tensors
-        T, H = x.shape
         grad = None
         for g in (dlogits32, dlogits):
             if g is not None:
                 grad = g.float() if grad is None else grad + g.float()
         if grad is None:
             return None, None, None
-        grad = grad.contiguous()
-        dev = x.device
-        code = _C.dtype_code(x.dtype)
-        dx, dw = torch.empty_like(x), torch.empty_like(w)
-        L = _C.lib()
-        ws_bytes = L.fmoe_router_prologue_backward_workspace_bytes(T, H, ctx.num_expert_keys, code)
-        ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
-        with torch.cuda.device(dev):
-            status = L.fmoe_router_prologue_backward(_C.ptr(grad), _C.ptr(x), _C.ptr(w), _C.ptr(stats), int(ctx.training), T, H,
-                                                     ctx.num_expert_keys, code, _C.ptr(dx), _C.ptr(dw), _C.ptr(ws), ws_bytes,
-                                                     _C.current_stream(dev))
-        _C.check(status, "router prologue backward")
+        dx, dw = router_prologue_backward(grad, x, w, stats, ctx.training)
         return dx, dw, None
+
+
+def router_prologue_backward(dlogits32: torch.Tensor, tokens: torch.Tensor, gate_weight: torch.Tensor, stats: torch.Tensor,
+                             training: bool):
+    """``(dtokens, dgate_weight)`` of ``logits = BatchNorm1d(tokens) @ gate_weight.T`` from the fp32 gradient of the logits
+    [T, 2*nk] and the forward's batch-norm statistics ``stats`` ([2*H] fp32: mean, 1/sqrt(var + eps));
+    ``fmoe_router_prologue_backward``."""
+    x, w, grad = tokens.contiguous(), gate_weight.contiguous(), dlogits32.contiguous()
+    T, H = x.shape
+    num_expert_keys = w.shape[0] // 2
+    if grad.shape != (T, 2 * num_expert_keys) or grad.dtype != torch.float32:
+        raise ValueError("expected an fp32 gradient of shape [T, 2*num_expert_keys]")
+    dev = _C.require_gpu(x, w, grad, stats)
+    code = _C.dtype_code(x.dtype)
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    L = _C.lib()
+    ws_bytes = L.fmoe_router_prologue_backward_workspace_bytes(T, H, num_expert_keys, code)
+    ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        status = L.fmoe_router_prologue_backward(_C.ptr(grad), _C.ptr(x), _C.ptr(w), _C.ptr(stats), int(training), T, H,
+                                                 num_expert_keys, code, _C.ptr(dx), _C.ptr(dw), _C.ptr(ws), ws_bytes,
+                                                 _C.current_stream(dev))
+    _C.check(status, "router prologue backward")
+    return dx, dw
+
+
+def route_backward(dgates: torch.Tensor, indices: torch.Tensor, logits32: torch.Tensor, num_expert_keys: int,
+                   norm_topk_prob: bool = False, dlogits: torch.Tensor = None) -> torch.Tensor:
+    """Gradient of the fp32 gate logits [T, 2*nk] from the gradient of the gates [T, K] (``fmoe_route_backward``): the
+    backward of per-half log-softmax, product-key top-k, exp and optional renormalisation
+    (flash_moe/modules/flash_moe.py:69-85) in one launch.  ``dlogits`` ([T, 2*nk] in the gates' dtype), the gradient of the
+    router logits the block returns, is added when given."""
+    if dgates.dim() != 2 or indices.shape != dgates.shape or indices.dtype != torch.int64:
+        raise ValueError("expected dgates [T, K] and int64 indices of the same shape")
+    T, K = dgates.shape
+    if logits32.shape != (T, 2 * num_expert_keys) or logits32.dtype != torch.float32:
+        raise ValueError("expected fp32 logits of shape [T, 2*num_expert_keys]")
+    if dlogits is not None and (dlogits.shape != logits32.shape or dlogits.dtype != dgates.dtype):
+        raise ValueError("dlogits must have the shape of the logits and the dtype of dgates")
+    dev = _C.require_gpu(dgates, indices, logits32, dlogits)
+    dg, idx, lg = dgates.contiguous(), indices.contiguous(), logits32.contiguous()
+    extra = dlogits.contiguous() if dlogits is not None else None
+    out = torch.empty_like(lg)
+    with torch.cuda.device(dev):
+        status = _C.lib().fmoe_route_backward(_C.ptr(dg), _C.ptr(idx), _C.ptr(lg), _C.ptr(extra), T, num_expert_keys, K,
+                                              _C.dtype_code(dg.dtype), int(bool(norm_topk_prob)), _C.ptr(out),
+                                              _C.current_stream(dev))
+    _C.check(status, "route backward")
+    return out
 
 
 def router_prologue(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.nn.BatchNorm1d):

@@ -217,6 +217,18 @@ int fmoe_pkm_forward(const void* values, const void* routing_weights, const int6
 int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64_t num_tokens, int num_keys, int top_k,
                               int dtype, void* drouter_logits, void* stream);
 
+/* Backward of the routing stage between the gate logits and the gates (flash_moe/modules/flash_moe.py:69-85: per-half
+ * log_softmax, flash_router_func, exp, optional renormalisation; autograd of torch ops around
+ * flash_moe/ops/triton/flash_router.py:317-344 in the reference), in one launch.
+ *   dgates [T, K] dtype: gradient of the gates; indices [T, K] int64 as returned by the forward (ids outside
+ *   [0, nk*nk) contribute nothing); logits_fp32 [T, 2*nk]: the fp32 gate logits the forward routed from
+ *   (router_logits_fp32 of fmoe_router_forward); dlogits_extra [T, 2*nk] dtype or NULL: gradient of the returned
+ *   router logits, added to the result; dlogits_fp32 [T, 2*nk] fp32, fully written: what
+ *   fmoe_router_prologue_backward takes.  num_keys <= 8192. */
+int fmoe_route_backward(const void* dgates, const int64_t* indices, const float* logits_fp32, const void* dlogits_extra,
+                        int64_t num_tokens, int num_keys, int top_k, int dtype, int norm_topk_prob, float* dlogits_fp32,
+                        void* stream);
+
 /* Backward of the router prologue q = BatchNorm1d(x), logits = q gate_w^T (flash_moe/modules/flash_moe.py:62-67; autograd of
  * torch ops in the reference).  The forward is fmoe_router_forward with top_k = 0: it leaves mean and 1/sqrt(var+eps), [2,H]
  * fp32, at byte offset fmoe_router_workspace_stats_offset() of its workspace; pass that as mean_rstd.

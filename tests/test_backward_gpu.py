@@ -43,6 +43,64 @@ def test_router_backward(dtype, T, nk, K):
     torch.testing.assert_close(got.double().sum(-1).cpu(), ref.sum(-1), rtol=5 * tol, atol=5 * tol * max(1.0, float(ref.abs().max())))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("norm", [False, True])
+@pytest.mark.parametrize("T,nk,K", [(64, 32, 16), (130, 128, 64), (9, 512, 128), (5, 8, 1)])
+def test_route_backward(dtype, norm, T, nk, K):
+    """Gate gradients -> gradient of the fp32 gate logits, against float64 autograd of log-softmax, pair sums, exp and
+    renormalisation on the same ids; ids out of range carry nothing; the gradient of the returned logits is added."""
+    from flash_moe.ops.hip.flash_router import route_backward
+
+    logits = torch.randn(T, 2 * nk, generator=gen(1)) * 2.0
+    idx = torch.stack([torch.randperm(nk * nk, generator=gen(10 + t))[:K] for t in range(T)])
+    if K > 2:
+        idx[::3, 1] = nk * nk + 7
+        idx[1::4, 2] = -1
+    dg = torch.randn(T, K, generator=gen(2)).to(dtype)
+    extra = (torch.randn(T, 2 * nk, generator=gen(3)) * 0.1).to(dtype)
+    valid = (idx >= 0) & (idx < nk * nk)
+    safe = idx.clamp(0, nk * nk - 1)
+    lg = logits.double().requires_grad_(True)
+    lp = torch.log_softmax(lg.view(T, 2, nk), -1)
+    e = (lp[:, 0].gather(1, safe // nk) + lp[:, 1].gather(1, safe % nk)).exp() * valid
+    gates = e / e.sum(-1, keepdim=True) if norm else e
+    ((gates * dg.double()).sum() + (lg * extra.double()).sum()).backward()
+    got = route_backward(dg.cuda(), idx.cuda(), logits.cuda(), nk, norm, extra.cuda())
+    assert got.dtype == torch.float32 and got.shape == (T, 2 * nk)
+    assert rel_fro(got, lg.grad) < 2e-5, rel_fro(got, lg.grad)
+    without = route_backward(dg.cuda(), idx.cuda(), logits.cuda(), nk, norm)
+    torch.testing.assert_close(without.cpu().double() + extra.double(), lg.grad, rtol=1e-4, atol=1e-5)
+    assert torch.equal(route_backward(dg.cuda(), idx.cuda(), logits.cuda(), nk, norm, extra.cuda()), got)
+
+
+@pytest.mark.parametrize("dtype,norm", [(torch.float32, False), (torch.float32, True), (torch.bfloat16, True)])
+def test_block_autograd_node_equals_the_composition_of_ops(dtype, norm):
+    """forward_autograd (one node, library calls only) and forward_autograd_ops (the reference's composition on the
+    differentiable per-op functions) give the same outputs and gradients."""
+    from test_block_gpu import build
+
+    m, _ = build(128, 256, 1024, 8, norm, dtype, seed=4, std=0.05)
+    x = torch.randn(2, 96, 128, generator=gen(5)).to(dtype).cuda()
+    wy = torch.randn(2, 96, 128, generator=gen(6)).cuda()
+    wl = (torch.randn(2, 192, 32, generator=gen(7)) * 0.1).cuda()
+    results = []
+    for fwd in (m.forward_autograd, m.forward_autograd_ops):
+        m.router_norm.reset_running_stats()
+        for p in m.parameters():
+            p.grad = None
+        xg = x.clone().requires_grad_(True)
+        y, logits = fwd(xg)
+        ((y.float() * wy).sum() + (logits.float() * wl).sum()).backward()
+        results.append((y.detach(), logits.detach(), xg.grad, {k: v.grad.clone() for k, v in m.named_parameters()}))
+    (y0, l0, gx0, gp0), (y1, l1, gx1, gp1) = results
+    tol = 2e-5 if dtype == torch.float32 else 1.5e-2
+    # same kernels for the logits; the gates come from the fused router here and from torch's exp there
+    assert torch.equal(l0, l1) and rel_fro(y0, y1) < tol
+    assert rel_fro(gx0, gx1) < tol, rel_fro(gx0, gx1)
+    for k in gp0:
+        assert rel_fro(gp0[k], gp1[k]) < tol, (k, rel_fro(gp0[k], gp1[k]))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(7, 64), (3, 5, 256), (128, 1024)])
 def test_swiglu_backward(dtype, shape):
