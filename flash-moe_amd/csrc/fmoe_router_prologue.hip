@@ -46,14 +46,28 @@ __global__ __launch_bounds__(kStatsThreads) void bn_partial_kernel(const T* __re
 #pragma unroll
     for (int v = 0; v < V; ++v) s1[v] = s2[v] = 0.0f;
     if (col_ok) {
-        for (int64_t r = r0 + wave; r < r1; r += 4) {
-            float xv[V];
-            unpack16<T>(*reinterpret_cast<const u32x4_t*>(x + r * hidden + col), xv);
+        // rows in batches of kBatch loads issued together (one memory round trip per batch); rows past the end are
+        // read from the last row and left out of the sums
+        constexpr int kBatch = 8;
+        for (int64_t rb = r0 + wave; rb < r1; rb += 4 * kBatch) {
+            u32x4_t raw[kBatch];
 #pragma unroll
-            for (int v = 0; v < V; ++v) {
-                const float d = xv[v] - pivot[v];
-                s1[v] += d;
-                s2[v] = __builtin_fmaf(d, d, s2[v]);
+            for (int i = 0; i < kBatch; ++i) {
+                const int64_t r = rb + 4 * i;
+                raw[i] = *reinterpret_cast<const u32x4_t*>(x + (r < r1 ? r : r1 - 1) * hidden + col);
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                if (rb + 4 * i < r1) {
+                    float xv[V];
+                    unpack16<T>(raw[i], xv);
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        const float d = xv[v] - pivot[v];
+                        s1[v] += d;
+                        s2[v] = __builtin_fmaf(d, d, s2[v]);
+                    }
+                }
             }
         }
     }
