@@ -151,15 +151,16 @@ extern "C" int fmoe_mlp_backward(const void* dy, const void* x, const void* gate
 
     rc = blas_gemm(kNN, T_, I, H, dy, H, down_w, I, dh, I, 0.0f, dtype, s);                        // dh = dy Wd
     if (rc) return rc;
-    rc = launch_swiglu_backward(dh, a, b, dab, dab + (size_t)I * elt, h, num_tokens, I, 2 * (int64_t)I, 2 * (int64_t)I, dtype, s);
+    char* db = dab + (size_t)num_tokens * I * elt;        // da and db as two dense [T, I] matrices
+    rc = launch_swiglu_backward(dh, a, b, dab, db, h, num_tokens, I, I, I, dtype, s);
     if (rc) return rc;
     rc = blas_gemm(kTN, H, I, T_, dy, H, h, I, ddown_w, I, 0.0f, dtype, s);                         // dWd = dy^T h
     if (rc) return rc;
-    rc = blas_gemm(kNN, T_, H, I, dab, 2 * I, gate_w, H, dx, H, 0.0f, dtype, s);                    // dx = da Wg
+    rc = blas_gemm(kNN, T_, H, I, dab, I, gate_w, H, dx, H, 0.0f, dtype, s);                        // dx = da Wg
     if (rc) return rc;
-    rc = blas_gemm(kNN, T_, H, I, dab + (size_t)I * elt, 2 * I, up_w, H, dx, H, 1.0f, dtype, s);    //    + db Wu
+    rc = blas_gemm(kNN, T_, H, I, db, I, up_w, H, dx, H, 1.0f, dtype, s);                           //    + db Wu
     if (rc) return rc;
-    rc = blas_gemm(kTN, I, H, T_, dab, 2 * I, x, H, dgate_w, H, 0.0f, dtype, s);                    // dWg = da^T x
+    rc = blas_gemm(kTN, I, H, T_, dab, I, x, H, dgate_w, H, 0.0f, dtype, s);                        // dWg = da^T x
     if (rc) return rc;
-    return blas_gemm(kTN, I, H, T_, dab + (size_t)I * elt, 2 * I, x, H, dup_w, H, 0.0f, dtype, s);  // dWu = db^T x
+    return blas_gemm(kTN, I, H, T_, db, I, x, H, dup_w, H, 0.0f, dtype, s);                         // dWu = db^T x
 }
