@@ -9,7 +9,8 @@ that is already resident in HBM.  The last line printed is one JSON object:
 
   value          tokens/s of the whole block (4096 tokens / mean step time over K steps)
   stages         mean duration of each launch of the block, measured with HIP events on the launch stream
-  roofline       the slowest kernel of the block against the roofline that bounds it
+  roofline       the slowest C-ABI call of the block (its kernels are named in `launches`) against the roofline
+                 that bounds it; rooflines_all has every call
   expert_c3      the routed-expert kernel alone on its own benchmark shape (16384 tokens), as HBM GB/s
   cpu_baseline   the CPU restatement of the reference's eager path (oracle/) on the same block, timed on
                  this machine's host cores
@@ -158,6 +159,16 @@ def stage_kernels(m, x):
     return fns, work, keep
 
 
+# kernels behind each timed C-ABI call, as they appear in the rocprofv3 summaries under profiles/
+LAUNCHES = {
+    "router_forward": ["bn_partial_kernel", "bn_finalize_kernel", "router_gate_kernel", "router_topk_kernel"],
+    "router_topk": ["router_topk_kernel"],
+    "expert": ["expert_prepare_kernel", "expert_scores_slice_kernel", "expert_gate_kernel", "expert_states_slice_kernel"],
+    "mlp_gate_up": ["gemm_dma_kernel<256x256 tiles, SwiGLU epilogue>"],
+    "mlp_down": ["gemm_dma_kernel<128x128 tiles, residual epilogue>"],
+}
+
+
 def roofline_entry(name, ms, w, traffic):
     if w["bound"] == "hbm":
         achieved = w["bytes"] / (ms * 1e-3) / 1e9
@@ -165,8 +176,8 @@ def roofline_entry(name, ms, w, traffic):
     else:
         achieved = w["flops"] / (ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
-    return dict(kernel=name, bound=w["bound"], achieved=round(achieved, 2), peak=peak, unit=unit,
-                frac=round(achieved / peak, 4), avg_launch_us=round(ms * 1e3, 2),
+    return dict(kernel=name, launches=LAUNCHES.get(name, [name]), bound=w["bound"], achieved=round(achieved, 2), peak=peak,
+                unit=unit, frac=round(achieved / peak, 4), avg_launch_us=round(ms * 1e3, 2),
                 algorithmic=w.get("bytes", w.get("flops")), traffic=traffic)
 
 
