@@ -60,51 +60,77 @@ __device__ inline uint64_t xor_lane_u64(uint64_t v, int mask, int lane) {
 }
 
 // Position of a key in the wave-wide sequence: p = lane*RK + r.
-// One compare-exchange layer of a bitonic network: partner = p ^ j, blocks of size k alternate direction.
-template <int RK, bool DESC>
-__device__ inline void bitonic_layer(uint64_t (&v)[RK], int lane, int k, int j) {
-    if (j < RK) {
+// One compare-exchange layer of a bitonic network: partner = p ^ J, blocks of size K alternate direction.
+// Which lanes keep the larger key is a function of the lane number alone, so it is a 64-bit compile-time constant per
+// (layer, register), handed to the selects as a lane mask (inverse ballot): no vector instruction and no live scalar
+// register per layer, where lane-number compares hoisted out of the token loop would be spilled.
+template <int RK> struct LaneMasks { uint64_t m[RK]; };
+template <int RK, int K, bool DESC> constexpr LaneMasks<RK> descending_block_lanes() {
+    LaneMasks<RK> out{};
+    for (int r = 0; r < RK; ++r)
+        for (int l = 0; l < kWave; ++l) out.m[r] |= (uint64_t)((((l * RK + r) & K) == 0) == DESC) << l;
+    return out;
+}
+template <int RK, int K, int J, bool DESC> constexpr LaneMasks<RK> keep_max_lanes() {
+    LaneMasks<RK> out{};
+    for (int r = 0; r < RK; ++r)
+        for (int l = 0; l < kWave; ++l) {
+            const int p = l * RK + r;
+            const bool desc_block = (((p & K) == 0) == DESC), first = (p & J) == 0;
+            out.m[r] |= (uint64_t)(first == desc_block) << l;
+        }
+    return out;
+}
+
+template <int RK, bool DESC, int K, int J>
+__device__ inline void bitonic_layer(uint64_t (&v)[RK], int lane) {
+    if constexpr (J < RK) {
+        constexpr LaneMasks<RK> desc = descending_block_lanes<RK, K, DESC>();
 #pragma unroll
         for (int r = 0; r < RK; ++r) {
-            if ((r & j) == 0) {
-                const int p = lane * RK + r;
-                const bool desc_block = (((p & k) == 0) == DESC);
-                const uint64_t a = v[r], b = v[r | j];
+            if ((r & J) == 0) {
+                const bool desc_block = __builtin_amdgcn_inverse_ballot_w64(desc.m[r]);
+                const uint64_t a = v[r], b = v[r | J];
                 const uint64_t hi = a > b ? a : b, lo = a > b ? b : a;
                 v[r] = desc_block ? hi : lo;
-                v[r | j] = desc_block ? lo : hi;
+                v[r | J] = desc_block ? lo : hi;
             }
         }
     } else {
-        const int m = j / RK;
+        constexpr LaneMasks<RK> keep = keep_max_lanes<RK, K, J, DESC>();
 #pragma unroll
         for (int r = 0; r < RK; ++r) {
-            const int p = lane * RK + r;
-            const uint64_t other = xor_lane_u64(v[r], m, lane);
-            const bool desc_block = (((p & k) == 0) == DESC);
-            const bool first = (p & j) == 0;
-            const bool keep_max = (first == desc_block);
+            const uint64_t other = xor_lane_u64(v[r], J / RK, lane);
+            const bool keep_max = __builtin_amdgcn_inverse_ballot_w64(keep.m[r]);
             // keep my key if it is the larger one and I keep the max, or the smaller one and I keep the min
             v[r] = ((v[r] > other) == keep_max) ? v[r] : other;
         }
     }
 }
 
+// layers J, J/2, ..., 1 of the stage with block size K
+template <int RK, bool DESC, int K, int J>
+__device__ inline void bitonic_stage(uint64_t (&v)[RK], int lane) {
+    bitonic_layer<RK, DESC, K, J>(v, lane);
+    if constexpr (J > 1) bitonic_stage<RK, DESC, K, J / 2>(v, lane);
+}
+// stages K, 2K, ..., N
+template <int RK, bool DESC, int K>
+__device__ inline void bitonic_stages_from(uint64_t (&v)[RK], int lane) {
+    bitonic_stage<RK, DESC, K, K / 2>(v, lane);
+    if constexpr (K < RK * kWave) bitonic_stages_from<RK, DESC, 2 * K>(v, lane);
+}
+
 template <int RK, bool DESC>
 __device__ inline void bitonic_sort(uint64_t (&v)[RK], int lane) {
-    constexpr int N = RK * kWave;
-#pragma unroll
-    for (int k = 2; k <= N; k <<= 1)
-#pragma unroll
-        for (int j = k >> 1; j >= 1; j >>= 1) bitonic_layer<RK, DESC>(v, lane, k, j);
+    bitonic_stages_from<RK, DESC, 2>(v, lane);
 }
 
 // v holds a bitonic sequence of N keys; sort it descending.
 template <int RK>
 __device__ inline void bitonic_merge_desc(uint64_t (&v)[RK], int lane) {
     constexpr int N = RK * kWave;
-#pragma unroll
-    for (int j = N >> 1; j >= 1; j >>= 1) bitonic_layer<RK, true>(v, lane, N, j);
+    bitonic_stage<RK, true, N, N / 2>(v, lane);
 }
 
 // Key at position `pos` of the wave-wide sequence (wave-uniform `pos`).
