@@ -421,6 +421,64 @@ __global__ __launch_bounds__(256) void prologue_bwd_prepare_kernel(const float* 
     }
 }
 
+// The same two tensors for the K-contiguous form of dWr = d^T q: d16 [T, N] as before (the A operand of dq = d Wr) plus the
+// transposes dT [N, T] and qT [H, T], written through a 64 x 64 LDS tile so that both sides of the kernel move 16-byte
+// packets.  Tile (tokens t0..t0+63) x (64 columns of q or of d); the column tiles of q come first.  Needs T, H and N to be
+// multiples of 64 and 16-bit elements.
+template <typename T>
+__global__ __launch_bounds__(256) void prologue_bwd_prepare_transposed_kernel(
+    const float* __restrict__ dlogits, const T* __restrict__ x, const float* __restrict__ mean_rstd, T* __restrict__ d16,
+    T* __restrict__ dT, T* __restrict__ qT, int64_t num_tokens, int hidden, int n_out) {
+    __shared__ T tile[64][64 + 2];          // [column][token], rows padded by one dword against bank conflicts
+    const int q_tiles = hidden / 64;
+    const int ct = (int)blockIdx.y;
+    const bool is_q = ct < q_tiles;
+    const int c0 = (is_q ? ct : ct - q_tiles) * 64;
+    const int64_t t0 = (int64_t)blockIdx.x * 64;
+    const int tid = (int)threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int idx = it * 256 + tid, r = idx >> 3, pk = idx & 7;      // token row r, packet pk (8 columns) of the tile
+        const int col = c0 + pk * 8;
+        float v[8];
+        if (is_q) {
+            float xv[8];
+            unpack16<T>(*reinterpret_cast<const u32x4_t*>(x + (t0 + r) * hidden + col), xv);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const f32x4_t m = *reinterpret_cast<const f32x4_t*>(mean_rstd + col + 4 * h);
+                const f32x4_t rs = *reinterpret_cast<const f32x4_t*>(mean_rstd + hidden + col + 4 * h);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[4 * h + j] = (xv[4 * h + j] - m[j]) * rs[j];
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const f32x4_t g = *reinterpret_cast<const f32x4_t*>(dlogits + (t0 + r) * n_out + col + 4 * h);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[4 * h + j] = g[j];
+            }
+            *reinterpret_cast<u32x4_t*>(d16 + (t0 + r) * n_out + col) = pack16<T>(v);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tile[pk * 8 + j][r] = Elem<T>::from_f32(v[j]);
+    }
+    __syncthreads();
+    T* out = is_q ? qT : dT;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int idx = it * 256 + tid, c = idx >> 3, pk = idx & 7;      // column c of the tile, tokens pk*8 .. pk*8+7
+        u32x4_t w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = __builtin_bit_cast(uint16_t, tile[c][pk * 8 + 2 * j]);
+            const uint32_t hi = __builtin_bit_cast(uint16_t, tile[c][pk * 8 + 2 * j + 1]);
+            w[j] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4_t*>(out + (int64_t)(c0 + c) * num_tokens + t0 + pk * 8) = w;
+    }
+}
+
 // partial: [row_blocks][2][H] = (sum dq, sum dq * xhat) over the block's rows; same geometry as bn_partial_kernel.
 template <typename T>
 __global__ __launch_bounds__(kStatsThreads) void bn_bwd_partial_kernel(const T* __restrict__ x, const T* __restrict__ dq,
@@ -535,7 +593,7 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(const T* __restrict__
 }
 
 struct PrologueBwdPlan {
-    size_t off_d16, off_q, off_dq, off_partial, off_sums, bytes;
+    size_t off_d16, off_dT, off_q, off_dq, off_partial, off_sums, bytes;
 };
 
 PrologueBwdPlan plan_prologue_backward(int64_t T_, int H, int nk, int dtype) {
@@ -544,6 +602,7 @@ PrologueBwdPlan plan_prologue_backward(int64_t T_, int H, int nk, int dtype) {
     size_t o = 0;
     auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
     p.off_d16 = take((size_t)T_ * 2 * nk * elt);
+    p.off_dT = take((size_t)T_ * 2 * nk * elt);
     p.off_q = take((size_t)T_ * H * elt);
     p.off_dq = take((size_t)T_ * H * elt);
     p.off_partial = take((size_t)kMaxRowBlocks * 2 * H * 4);
@@ -564,10 +623,24 @@ int launch_prologue_backward(const float* dlogits, const void* x, const void* ga
     const int N = 2 * nk;
     const int widest = H > N ? H : N;
     const int col_blocks = (widest / V + 255) / 256;
-    hipLaunchKernelGGL((prologue_bwd_prepare_kernel<T>), dim3((unsigned)(T_ * col_blocks)), dim3(256), 0, s, dlogits,
-                       (const T*)x, mean_rstd, d16, q, H, N, col_blocks);
-    FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(prepare)");
-    if (int rc = blas_gemm(kBlasTN, N, H, (int)T_, d16, N, q, H, dgate_w, H, 0.0f, dtype, s)) return rc;      // dWr = d^T q
+    bool transposed = false;
+    if constexpr (sizeof(T) == 2) {
+        if (T_ % 64 == 0 && H % 64 == 0 && N % 64 == 0) {
+            // dWr[N, H] = dT[N, T] qT[H, T]^T: both operands K-contiguous, the forward's own GEMM ("down" form)
+            T* dT = (T*)(ws + p.off_dT);
+            hipLaunchKernelGGL((prologue_bwd_prepare_transposed_kernel<T>), dim3((unsigned)(T_ / 64), (unsigned)((H + N) / 64)),
+                               dim3(256), 0, s, dlogits, (const T*)x, mean_rstd, d16, dT, q, T_, H, N);
+            FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(prepare)");
+            if (int rc = fmoe_mlp_down(dT, q, N, H, (int)T_, dtype, nullptr, dgate_w, s)) return rc;
+            transposed = true;
+        }
+    }
+    if (!transposed) {
+        hipLaunchKernelGGL((prologue_bwd_prepare_kernel<T>), dim3((unsigned)(T_ * col_blocks)), dim3(256), 0, s, dlogits,
+                           (const T*)x, mean_rstd, d16, q, H, N, col_blocks);
+        FMOE_CHECK_LAUNCH("fmoe_router_prologue_backward(prepare)");
+        if (int rc = blas_gemm(kBlasTN, N, H, (int)T_, d16, N, q, H, dgate_w, H, 0.0f, dtype, s)) return rc;      // dWr = d^T q
+    }
     if (int rc = blas_gemm(kBlasNN, (int)T_, H, N, d16, N, gate_w, H, dq, H, 0.0f, dtype, s)) return rc;       // dq = d Wr
     if (training) {
         const int strips = (H + kWave * V - 1) / (kWave * V);

@@ -354,7 +354,7 @@ def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("training", [True, False])
-@pytest.mark.parametrize("T,H,nk", [(256, 128, 16), (1000, 1024, 128), (65, 64, 8)])
+@pytest.mark.parametrize("T,H,nk", [(256, 128, 16), (1000, 1024, 128), (65, 64, 8), (256, 128, 32), (1024, 1024, 128)])
 def test_router_prologue_backward(dtype, training, T, H, nk):
     """Batch norm + gate product: gradients of the input and of the gate weights against float64 autograd."""
     from flash_moe.ops.hip.flash_router import router_prologue
