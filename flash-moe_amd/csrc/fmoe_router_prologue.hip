@@ -410,14 +410,19 @@ __global__ __launch_bounds__(256) void prologue_bwd_prepare_kernel(const float* 
     }
     if (col < n_out) {
         const int64_t at = (int64_t)row * n_out + col;
-        float dv[V];
+        if (n_out % V == 0) {
+            float dv[V];
 #pragma unroll
-        for (int h = 0; h < V / 4; ++h) {
-            const f32x4_t g = *reinterpret_cast<const f32x4_t*>(dlogits + at + 4 * h);
+            for (int h = 0; h < V / 4; ++h) {
+                const f32x4_t g = *reinterpret_cast<const f32x4_t*>(dlogits + at + 4 * h);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) dv[4 * h + j] = g[j];
+                for (int j = 0; j < 4; ++j) dv[4 * h + j] = g[j];
+            }
+            *reinterpret_cast<u32x4_t*>(d16 + at) = pack16<T>(dv);
+        } else {
+            // rows of d that are not a whole number of 16-byte packets (2*nk not a multiple of V): element by element
+            for (int j = 0; j < V && col + j < n_out; ++j) d16[at + j] = Elem<T>::from_f32(dlogits[at + j]);
         }
-        *reinterpret_cast<u32x4_t*>(d16 + at) = pack16<T>(dv);
     }
 }
 
@@ -622,7 +627,7 @@ int launch_prologue_backward(const float* dlogits, const void* x, const void* ga
     float *partial = (float*)(ws + p.off_partial), *sums = (float*)(ws + p.off_sums);
     const int N = 2 * nk;
     const int widest = H > N ? H : N;
-    const int col_blocks = (widest / V + 255) / 256;
+    const int col_blocks = ((widest + V - 1) / V + 255) / 256;
     bool transposed = false;
     if constexpr (sizeof(T) == 2) {
         if (T_ % 64 == 0 && H % 64 == 0 && N % 64 == 0) {
@@ -771,8 +776,8 @@ extern "C" int fmoe_router_prologue_backward(const float* dlogits_fp32, const vo
     FMOE_REQUIRE(num_tokens > 0 && hidden > 0 && num_keys > 0 && num_tokens < (1ll << 24), FMOE_ERR_BAD_SHAPE,
                  "fmoe_router_prologue_backward: bad shape T=%lld H=%d nk=%d", (long long)num_tokens, hidden, num_keys);
     const int vec = (int)(16 / dtype_size(dtype));
-    FMOE_REQUIRE(hidden % vec == 0 && (2 * num_keys) % vec == 0, FMOE_ERR_ALIGNMENT,
-                 "fmoe_router_prologue_backward: hidden=%d and 2*num_keys=%d must be multiples of %d", hidden, 2 * num_keys, vec);
+    FMOE_REQUIRE(hidden % vec == 0, FMOE_ERR_ALIGNMENT,
+                 "fmoe_router_prologue_backward: hidden=%d must be a multiple of %d", hidden, vec);
     FMOE_REQUIRE(dlogits_fp32 && x && gate_w && mean_rstd && dx && dgate_w, FMOE_ERR_NULL_POINTER,
                  "fmoe_router_prologue_backward: null tensor pointer");
     FMOE_REQUIRE(aligned16(x) && aligned16(dx) && aligned16(dlogits_fp32) && aligned16(mean_rstd), FMOE_ERR_ALIGNMENT,

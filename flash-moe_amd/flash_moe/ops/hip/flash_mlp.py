@@ -126,7 +126,11 @@ class FlashMLPFunc(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def forward(ctx, x, gate_weight, up_weight, down_weight):
-        if not any(ctx.needs_input_grad) or x.numel() == 0:
+        if not any(ctx.needs_input_grad):
+            return mlp_forward(x, gate_weight, up_weight, down_weight)
+        if x.numel() == 0:
+            # nothing to keep for an empty batch: the backward returns zero gradients of the right shapes
+            ctx.save_for_backward(x, gate_weight, up_weight, down_weight)
             return mlp_forward(x, gate_weight, up_weight, down_weight)
         out, saved = mlp_forward_saving(x, gate_weight, up_weight, down_weight)
         ctx.save_for_backward(x, gate_weight, up_weight, down_weight, saved)
@@ -135,8 +139,8 @@ class FlashMLPFunc(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def backward(ctx, dout):
-        x, gate_weight, up_weight, down_weight, saved = ctx.saved_tensors
-        return mlp_backward(dout, x, gate_weight, up_weight, down_weight, saved)
+        x, gate_weight, up_weight, down_weight, *rest = ctx.saved_tensors
+        return mlp_backward(dout, x, gate_weight, up_weight, down_weight, rest[0] if rest else None)
 
 
 def flash_mlp_func(x: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor, down_weight: torch.Tensor) -> torch.Tensor:

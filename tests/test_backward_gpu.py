@@ -336,6 +336,55 @@ def test_backward_of_empty_batches():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_autograd_of_an_empty_batch_gives_zero_gradients(dtype):
+    """An empty batch with trainable parameters: the autograd functions return zero gradients of the right shapes."""
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+    from flash_moe.ops.hip.flash_mlp import flash_mlp_func
+
+    H, I = 64, 128
+    wg, wu, wd = (torch.randn(s, device="cuda").to(dtype).requires_grad_(True) for s in ((I, H), (I, H), (H, I)))
+    x = torch.zeros(0, H, device="cuda", dtype=dtype, requires_grad=True)
+    y = flash_mlp_func(x, wg, wu, wd)
+    assert y.shape == (0, H)
+    y.sum().backward()
+    assert x.grad.shape == (0, H) and all(w.grad is not None and (w.grad == 0).all() for w in (wg, wu, wd))
+
+    m = FlashMoE(FlashMoEConfig(H, I, "silu", 64, 4, False)).to(device="cuda", dtype=dtype).eval()
+    out, logits = m(torch.zeros(1, 0, H, device="cuda", dtype=dtype))
+    assert out.shape == (1, 0, H) and logits.shape == (2, 0, 8)
+    (out.float().sum() + logits.float().sum()).backward()
+    for name, p in m.named_parameters():
+        assert p.grad is None or (p.grad == 0).all(), name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_backward_with_a_key_count_that_is_not_a_multiple_of_four(dtype):
+    """num_experts = 100 -> 10 keys per half: rows of the gate gradient are not whole 16-byte packets."""
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+
+    H, I, E, K, T = 64, 128, 100, 4, 96
+    m = FlashMoE(FlashMoEConfig(H, I, "silu", E, K, True)).to(device="cuda", dtype=dtype)
+    x = torch.randn(2, T // 2, H, generator=gen(3)).to(dtype).cuda()
+
+    def grads(forward):
+        for p in m.parameters():
+            p.grad = None
+        m.router_norm.reset_running_stats()
+        xg = x.clone().requires_grad_(True)
+        y, logits = forward(xg)
+        (y.float().square().sum() + logits.float().sum() * 0.01).backward()
+        return xg.grad, {k: v.grad.clone() for k, v in m.named_parameters()}
+
+    gx, gp = grads(m.forward_autograd)
+    gx2, gp2 = grads(m.forward_autograd_ops)
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    assert torch.isfinite(gx).all() and rel_fro(gx, gx2) < tol
+    for k in gp:
+        assert torch.isfinite(gp[k]).all() and rel_fro(gp[k], gp2[k]) < tol, k
+    assert gp["router_gate.weight"].shape == (20, H) and gp["router_gate.weight"].abs().sum() > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
     from flash_moe.ops.hip.flash_mlp import mlp_backward, mlp_forward, mlp_forward_saving
 
@@ -354,7 +403,8 @@ def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("training", [True, False])
-@pytest.mark.parametrize("T,H,nk", [(256, 128, 16), (1000, 1024, 128), (65, 64, 8), (256, 128, 32), (1024, 1024, 128)])
+@pytest.mark.parametrize("T,H,nk", [(256, 128, 16), (1000, 1024, 128), (65, 64, 8), (256, 128, 32), (1024, 1024, 128),
+                                    (128, 64, 10), (70, 64, 6), (64, 128, 30), (40, 32, 81)])
 def test_router_prologue_backward(dtype, training, T, H, nk):
     """Batch norm + gate product: gradients of the input and of the gate weights against float64 autograd."""
     from flash_moe.ops.hip.flash_router import router_prologue

@@ -195,7 +195,10 @@ def test_fused_router_eval_mode_and_normalised_gates():
     (logits, scores, indices, gates, logits32), bn = _fused(x, wr, nk, K, True, torch.float32, training=False, rm=rm, rv=rv)
     ref_logits, ref_lp = orc.router_prologue(x, wr, nk, rm.clone(), rv.clone(), training=False)
     torch.testing.assert_close(logits.cpu().view(T, 2, nk).transpose(0, 1), ref_logits, rtol=1e-4, atol=1e-4)
-    torch.testing.assert_close(bn.running_mean.cpu(), rm) and int(bn.num_batches_tracked) == 0   # untouched in eval mode
+    # the buffers are untouched in eval mode
+    torch.testing.assert_close(bn.running_mean.cpu(), rm, rtol=0, atol=0)
+    torch.testing.assert_close(bn.running_var.cpu(), rv, rtol=0, atol=0)
+    assert int(bn.num_batches_tracked) == 0
     torch.testing.assert_close(gates.sum(-1).cpu(), torch.ones(T), rtol=1e-5, atol=1e-5)
     o_s, o_i = orc.router_topk(ref_lp, nk, K)
     overlap = sum(len(set(a.tolist()) & set(b.tolist())) for a, b in zip(indices.cpu(), o_i)) / o_i.numel()
