@@ -14,15 +14,51 @@
 //   router_topk_kernel  (fmoe_router.hip)
 #include <math.h>
 
+#include <mutex>
+
 #include "fmoe_common.h"
 #include "fmoe_mfma.h"
 #include "fmoe_vec.h"
+
+// Scratch of fmoe_router_forward_noalloc: the batch-norm partials and the mean / 1/std vectors of one call, for hidden sizes
+// up to kNoAllocMaxHidden.  Every GPU the library runs on holds its own copy at its own address for the life of the
+// process; host code reaches it only through the address hipGetSymbolAddress returns for the current device.
+#define FMOE_NOALLOC_MAX_HIDDEN 2048
+#define FMOE_NOALLOC_SCRATCH_BYTES (256 * 3 * FMOE_NOALLOC_MAX_HIDDEN * 4 + 2 * FMOE_NOALLOC_MAX_HIDDEN * 4)
+static __device__ __align__(256) unsigned char scratch[FMOE_NOALLOC_SCRATCH_BYTES];
 
 namespace fmoe {
 namespace {
 
 constexpr int kStatsThreads = 256;
 constexpr int kMaxRowBlocks = 256;
+static_assert(kMaxRowBlocks * 3 * FMOE_NOALLOC_MAX_HIDDEN * 4 % 256 == 0, "the static scratch holds the largest plan exactly");
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("fmoe_router_forward_noalloc: no usable current device (%s)", hipGetErrorString(e));
+        return e != hipSuccess ? (int)e : FMOE_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            set_error("fmoe_router_forward_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return e != hipSuccess ? (int)e : FMOE_ERR_UNSUPPORTED;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return FMOE_OK;
+}
 
 // Block (rb, strip): rows [rb*rows_per_block, ...), columns strip*64*V + lane*V .. +V; the 4 waves take rows 4 apart.
 // Sums are taken relative to the block's first row (pivot) so that var = E[d^2] - E[d]^2 does not cancel.
@@ -681,6 +717,27 @@ extern "C" int fmoe_router_forward(const void* x, const void* gate_w, void* runn
                                      momentum, eps, num_tokens, hidden, num_keys, top_k, dtype, norm_topk_prob,
                                      router_logits, logits_fp32, scores, indices, gates, nullptr, 0u, workspace,
                                      workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running_mean, void* running_var,
+                                           int64_t* num_batches_tracked, int stats_dtype, int training, float momentum,
+                                           float eps, int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype,
+                                           int norm_topk_prob, void* router_logits, float* logits_fp32, float* scores,
+                                           int64_t* indices, void* gates, void* stream) {
+    using namespace fmoe;
+    clear_error();
+    FMOE_REQUIRE(hidden <= FMOE_NOALLOC_MAX_HIDDEN, FMOE_ERR_UNSUPPORTED,
+                 "fmoe_router_forward_noalloc: hidden=%d exceeds the %d columns its static scratch is sized for; use "
+                 "fmoe_router_forward with a workspace", hidden, FMOE_NOALLOC_MAX_HIDDEN);
+    if (num_tokens <= 0 || hidden <= 0 || num_keys <= 0)   // rejected (or empty) below, before any scratch is needed
+        return router_forward_impl(x, gate_w, running_mean, running_var, num_batches_tracked, stats_dtype, training, momentum,
+                                   eps, num_tokens, hidden, num_keys, top_k, dtype, norm_topk_prob, router_logits, logits_fp32,
+                                   scores, indices, gates, nullptr, 0u, nullptr, 0, (hipStream_t)stream);
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return router_forward_impl(x, gate_w, running_mean, running_var, num_batches_tracked, stats_dtype, training, momentum,
+                               eps, num_tokens, hidden, num_keys, top_k, dtype, norm_topk_prob, router_logits, logits_fp32,
+                               scores, indices, gates, nullptr, 0u, ws, (size_t)FMOE_NOALLOC_SCRATCH_BYTES, (hipStream_t)stream);
 }
 
 int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_mean, void* running_var,

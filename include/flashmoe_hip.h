@@ -95,6 +95,18 @@ int fmoe_router_forward(const void* x, const void* gate_w, void* running_mean, v
                         void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* fmoe_router_forward for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same results.  It has no
+ * counterpart in the reference.  The scratch the call needs (batch-norm partials, mean and 1/std: about 6 MiB) is a
+ * static array in device memory, one copy per GPU for the life of the process, so hidden is limited to 2048
+ * (FMOE_ERR_UNSUPPORTED beyond) and two calls that overlap on one GPU (different streams or threads) race on it.
+ * The call itself allocates and frees nothing; the device the stream belongs to must be the current device. */
+int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running_mean, void* running_var,
+                                int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
+                                int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
+                                void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
+                                void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Routed experts.
  * Replaces triton_flash_expert_func / FlashExpertFunc.forward / _flash_expert_forward and its host-side
