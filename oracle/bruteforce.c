@@ -154,3 +154,48 @@ int bf_mlp(const double* x, const double* wg, const double* wu, const double* wd
     free(hbuf);
     return 0;
 }
+
+/* Expert-centric bucketing by exhaustive scan: for every expert in turn, every pair in index order.
+ * idx: [P] expert id of pair p; offsets: [E+1]; sorted_pairs: [P] (the first offsets[E] entries are written).
+ * Ids outside [0,E) belong to no segment. */
+int bf_bucket(const int64_t* idx, int64_t P, int64_t E, int32_t* offsets, int32_t* sorted_pairs) {
+    int64_t n = 0;
+    for (int64_t e = 0; e < E; ++e) {
+        offsets[e] = (int32_t)n;
+        for (int64_t p = 0; p < P; ++p)
+            if (idx[p] == e) sorted_pairs[n++] = (int32_t)p;
+    }
+    offsets[E] = (int32_t)n;
+    return 0;
+}
+
+/* PEER: bf_expert with the erf GELU in place of SiLU.  PKM: out[t] = sum_k w[t,k] * values[idx[t,k]]. */
+int bf_peer(const double* x, const double* wd, const double* wu, const int64_t* idx,
+            const double* g, int64_t T, int H, int64_t E, int K, double* out) {
+    for (int64_t t = 0; t < T; ++t) {
+        double* o = out + t * H;
+        for (int h = 0; h < H; ++h) o[h] = 0.0;
+        for (int k = 0; k < K; ++k) {
+            int64_t e = idx[t * K + k];
+            if (e < 0 || e >= E) return -1;
+            double s = 0.0;
+            for (int h = 0; h < H; ++h) s += x[t * H + h] * wd[e * H + h];
+            double a = 0.5 * s * (1.0 + erf(s / sqrt(2.0))) * g[t * K + k];
+            for (int h = 0; h < H; ++h) o[h] += a * wu[e * H + h];
+        }
+    }
+    return 0;
+}
+
+int bf_pkm(const double* values, const int64_t* idx, const double* w, int64_t T, int H, int64_t E, int K, double* out) {
+    for (int64_t t = 0; t < T; ++t) {
+        double* o = out + t * H;
+        for (int h = 0; h < H; ++h) o[h] = 0.0;
+        for (int k = 0; k < K; ++k) {
+            int64_t e = idx[t * K + k];
+            if (e < 0 || e >= E) return -1;
+            for (int h = 0; h < H; ++h) o[h] += w[t * K + k] * values[e * H + h];
+        }
+    }
+    return 0;
+}

@@ -21,7 +21,7 @@ def _load():
         if not os.path.exists(_LIB_PATH):
             raise RuntimeError(f"{_LIB_PATH} missing: run `make -C oracle` (or __graft_entry__.build())")
         _lib = ctypes.CDLL(_LIB_PATH)
-        for name in ("bf_router_topk", "bf_prologue", "bf_expert", "bf_mlp"):
+        for name in ("bf_router_topk", "bf_prologue", "bf_expert", "bf_mlp", "bf_bucket", "bf_peer", "bf_pkm"):
             getattr(_lib, name).restype = ctypes.c_int
     return _lib
 
@@ -81,4 +81,39 @@ def mlp(x, wg, wu, wd):
                         ctypes.c_int(wg.shape[0]), _p(out))
     if rc:
         raise ValueError(f"bf_mlp failed: {rc}")
+    return out
+
+
+def bucket(idx: np.ndarray, num_experts: int):
+    """idx [P] int64 -> (expert_offsets [E+1] int32, sorted_pair_ids [offsets[E]] int32) by exhaustive scan."""
+    idx = np.ascontiguousarray(idx, dtype=np.int64).reshape(-1)
+    offsets = np.empty(num_experts + 1, np.int32)
+    pairs = np.empty(max(idx.size, 1), np.int32)
+    rc = _load().bf_bucket(_p(idx), ctypes.c_int64(idx.size), ctypes.c_int64(num_experts), _p(offsets), _p(pairs))
+    if rc:
+        raise ValueError(f"bf_bucket failed: {rc}")
+    return offsets, pairs[: offsets[-1]]
+
+
+def peer(x, wd, wu, idx, g):
+    x, wd, wu, g = (np.ascontiguousarray(a, dtype=np.float64) for a in (x, wd, wu, g))
+    idx = np.ascontiguousarray(idx, dtype=np.int64)
+    T, H = x.shape
+    out = np.empty((T, H), np.float64)
+    rc = _load().bf_peer(_p(x), _p(wd), _p(wu), _p(idx), _p(g), ctypes.c_int64(T), ctypes.c_int(H),
+                         ctypes.c_int64(wd.shape[0]), ctypes.c_int(idx.shape[1]), _p(out))
+    if rc:
+        raise ValueError(f"bf_peer failed: {rc}")
+    return out
+
+
+def pkm(values, idx, w):
+    values, w = (np.ascontiguousarray(a, dtype=np.float64) for a in (values, w))
+    idx = np.ascontiguousarray(idx, dtype=np.int64)
+    T, H = idx.shape[0], values.shape[1]
+    out = np.empty((T, H), np.float64)
+    rc = _load().bf_pkm(_p(values), _p(idx), _p(w), ctypes.c_int64(T), ctypes.c_int(H), ctypes.c_int64(values.shape[0]),
+                        ctypes.c_int(idx.shape[1]), _p(out))
+    if rc:
+        raise ValueError(f"bf_pkm failed: {rc}")
     return out

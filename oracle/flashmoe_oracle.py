@@ -17,6 +17,11 @@ term, a wrong sign or a transposed operand fails a test that does not retype the
 * ``expert_forward``    float64 loop implementation in ``oracle/bruteforce.c``; special cases
                         (zero gates, one expert repeated, linearity in the gates, permutation of k).
 * ``mlp_forward``       float64 loop implementation in ``oracle/bruteforce.c``.
+* ``expert_bucketing``  exhaustive C scan in ``oracle/bruteforce.c`` (for every expert, every pair in index
+                        order), invariants (offsets monotone, ``offsets[E]`` = number of valid pairs, each
+                        segment one expert, the pairs a permutation), a numpy ``argsort(kind="stable")``.
+* ``peer_forward``, ``pkm_forward``   float64 loops in ``oracle/bruteforce.c`` (``erf`` of the C library),
+                        closed forms (a unit weight copies a row; gelu(s) - gelu(-s) = s).
 * ``block_forward``     composition of the above; equality with calling the stages one by one.
 
 The reference holds no golden vectors or asserting tests for this path (its tests only print),
@@ -124,6 +129,53 @@ def expert_forward(
         a = F.silu(s) * weights[lo:hi]
         out[lo:hi] = torch.matmul(a.unsqueeze(-2), wu).squeeze(-2)
     return out
+
+
+def expert_bucketing(indices: torch.Tensor, num_experts: int):
+    """Token-centric (token, expert) pairs -> expert-centric segments.
+
+    Follows ``_preprocess_expert_centric_indices_pytorch`` (flash_moe/ops/triton/flash_expert.py:528-577): flatten
+    the pairs, sort them by expert id, permute the token ids, ``bincount`` + ``cumsum`` into ``expert_offsets``.
+    Returns ``(sorted_token_ids int32 [P'], expert_offsets int32 [E+1], sorted_pair_ids int32 [P'],
+    sorted_expert_ids int32 [P'])``.  Two points the reference leaves open are fixed here: the sort is stable
+    (``torch.sort`` there is not), so a segment lists its pairs in ascending pair index, the canonical order every
+    comparison uses; and ids outside ``[0, num_experts)`` are dropped (P' = number of valid pairs), where the
+    reference would index out of bounds.
+    """
+    num_tokens, top_k = indices.shape
+    expert_ids = indices.reshape(-1)
+    valid = (expert_ids >= 0) & (expert_ids < num_experts)
+    pair_ids = torch.arange(num_tokens * top_k, dtype=torch.int64)[valid]
+    order = torch.sort(expert_ids[valid], stable=True)
+    sorted_pair_ids = pair_ids[order.indices]
+    sorted_token_ids = sorted_pair_ids // max(top_k, 1)
+    counts = torch.bincount(order.values, minlength=num_experts)
+    offsets = torch.zeros(num_experts + 1, dtype=torch.int32)
+    offsets[1:] = torch.cumsum(counts, dim=0)
+    return sorted_token_ids.int(), offsets, sorted_pair_ids.int(), order.values.int()
+
+
+def peer_forward(hidden, down_table, up_table, weights, indices):
+    """PEER: ``out[t] = sum_k gelu(<x_t, Wd[idx[t,k]]>) * w[t,k] * Wu[idx[t,k]]`` with the erf GELU.
+
+    Follows the eager form of the reference's test (tests/test_peer.py:9-24): two embedding gathers, a batched
+    mat-vec, ``F.gelu`` (exact, erf), the routing weight, a batched vec-mat; note the argument order (weights
+    before indices) of ``triton_peer_func`` (flash_moe/ops/triton/peer.py:246-255).
+    """
+    wd = F.embedding(indices, down_table)
+    wu = F.embedding(indices, up_table)
+    s = torch.matmul(wd, hidden.unsqueeze(-1)).squeeze(-1)
+    a = F.gelu(s) * weights
+    return torch.matmul(a.unsqueeze(-2), wu).squeeze(-2)
+
+
+def pkm_forward(values, weights, indices):
+    """Product-key memory read-out ``out[t] = sum_k w[t,k] * values[idx[t,k]]``.
+
+    Follows tests/test_pkm.py:9-20 (an embedding-bag with per-sample weights) and ``triton_pkm_func``
+    (flash_moe/ops/triton/pkm.py:195-200).
+    """
+    return torch.matmul(weights.unsqueeze(-2), F.embedding(indices, values)).squeeze(-2)
 
 
 def mlp_forward(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor) -> torch.Tensor:

@@ -219,3 +219,87 @@ def test_block_bruteforce_end_to_end():
     y = bf.mlp(x[0].numpy(), w.gate_proj.numpy(), w.up_proj.numpy(), w.down_proj.numpy()) + bf.expert(
         x[0].numpy(), w.down_embed.numpy(), w.up_embed.numpy(), order, gates)
     np.testing.assert_allclose(r["y"][0].numpy(), y, rtol=1e-9, atol=1e-11)
+
+
+# ----------------------------------------------------------------------------------------------
+# expert-centric bucketing (flash_expert.py:528-577)
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,K,E,seed", [(40, 4, 16, 0), (7, 5, 100, 1), (64, 8, 8, 2), (1, 1, 3, 3), (33, 3, 1, 4)])
+def test_bucketing_matches_exhaustive_scan(T, K, E, seed):
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.randint(0, E, (T, K), generator=g)
+    if T > 4:
+        idx[1, 0] = -3          # ids outside [0, E) belong to no segment
+        idx[2, K - 1] = E + 5
+    tok, offsets, pairs, experts = orc.expert_bucketing(idx, E)
+    b_offsets, b_pairs = bf.bucket(idx.numpy(), E)
+    np.testing.assert_array_equal(offsets.numpy(), b_offsets)
+    np.testing.assert_array_equal(pairs.numpy(), b_pairs)          # stable: ascending pair index inside a segment
+    np.testing.assert_array_equal(tok.numpy(), b_pairs // K)
+    np.testing.assert_array_equal(experts.numpy(), idx.reshape(-1).numpy()[b_pairs])
+    assert offsets.dtype == torch.int32 and pairs.dtype == torch.int32 and tok.dtype == torch.int32
+
+
+def test_bucketing_invariants_and_numpy_argsort():
+    g = torch.Generator().manual_seed(9)
+    T, K, E = 500, 16, 300
+    idx = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    tok, offsets, pairs, experts = orc.expert_bucketing(idx, E)
+    flat = idx.reshape(-1).numpy()
+    P = T * K
+    assert int(offsets[0]) == 0 and int(offsets[-1]) == P and (offsets[1:] >= offsets[:-1]).all()
+    assert sorted(pairs.tolist()) == list(range(P))                 # a permutation: the multiset of pairs is preserved
+    for e in (0, 1, E // 2, E - 1):                                 # each segment holds one expert, in ascending pair index
+        seg = pairs[int(offsets[e]):int(offsets[e + 1])].numpy()
+        assert (flat[seg] == e).all() and (np.diff(seg) > 0).all()
+    np.testing.assert_array_equal(pairs.numpy(), np.argsort(flat, kind="stable").astype(np.int32))
+    np.testing.assert_array_equal(np.diff(offsets.numpy()), np.bincount(flat, minlength=E))
+    # one expert selected by every token: a single segment listing the tokens in order
+    one = torch.full((T, 1), 7)
+    tok1, off1, pairs1, _ = orc.expert_bucketing(one, E)
+    assert tok1.tolist() == list(range(T)) and int(off1[7]) == 0 and int(off1[8]) == T and int(off1[-1]) == T
+    # no pairs at all
+    tok0, off0, pairs0, _ = orc.expert_bucketing(torch.zeros(0, 4, dtype=torch.int64), 5)
+    assert tok0.numel() == 0 and off0.tolist() == [0] * 6
+
+
+# ----------------------------------------------------------------------------------------------
+# PEER / PKM (tests/test_peer.py:9-24, tests/test_pkm.py:9-20)
+# ----------------------------------------------------------------------------------------------
+def test_peer_and_pkm_match_bruteforce():
+    T, H, E, K = 24, 20, 50, 6
+    x, wd, wu, idx, w = orc.make_expert_inputs(T, H, E, K, seed=12, std=0.7)
+    x, wd, wu, w = (t.double() for t in (x, wd, wu, w))
+    np.testing.assert_allclose(orc.peer_forward(x, wd, wu, w, idx).numpy(),
+                               bf.peer(x.numpy(), wd.numpy(), wu.numpy(), idx.numpy(), w.numpy()), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(orc.pkm_forward(wu, w, idx).numpy(), bf.pkm(wu.numpy(), idx.numpy(), w.numpy()),
+                               rtol=1e-12, atol=1e-13)
+    # the erf GELU is neither SiLU nor the tanh approximation
+    silu = orc.expert_forward(x, wd, wu, idx, w)
+    assert (orc.peer_forward(x, wd, wu, w, idx) - silu).abs().max() > 1e-3
+
+
+def test_peer_and_pkm_closed_forms():
+    g = torch.Generator().manual_seed(13)
+    T, H, E = 9, 12, 30
+    values = torch.randn(E, H, generator=g, dtype=torch.float64)
+    idx = torch.randint(0, E, (T, 1), generator=g)
+    # PKM: a unit weight copies the row; zero weights give zero; the same row twice doubles it
+    assert torch.equal(orc.pkm_forward(values, torch.ones(T, 1, dtype=torch.float64), idx), values[idx[:, 0]])
+    assert orc.pkm_forward(values, torch.zeros(T, 1, dtype=torch.float64), idx).abs().max() == 0
+    twice = orc.pkm_forward(values, torch.ones(T, 2, dtype=torch.float64), idx.expand(T, 2))
+    torch.testing.assert_close(twice, 2 * values[idx[:, 0]], rtol=1e-14, atol=0)
+    # PEER: gelu(s) - gelu(-s) = s, so x and -x on the same expert differ by s * w * up[e]
+    x = torch.randn(T, H, generator=g, dtype=torch.float64)
+    wd = torch.randn(E, H, generator=g, dtype=torch.float64) * 0.5
+    w = torch.rand(T, 1, generator=g, dtype=torch.float64) + 0.1
+    s = (x * wd[idx[:, 0]]).sum(-1, keepdim=True)
+    diff = orc.peer_forward(x, wd, values, w, idx) - orc.peer_forward(-x, wd, values, w, idx)
+    torch.testing.assert_close(diff, s * w * values[idx[:, 0]], rtol=1e-12, atol=1e-13)
+    # gelu(0) = 0: a zero input row gives a zero output row, whatever the weights
+    assert orc.peer_forward(torch.zeros(T, H, dtype=torch.float64), wd, values, w, idx).abs().max() == 0
+    # known values of the erf GELU: gelu(1) = 0.5 * (1 + erf(1/sqrt 2)) = 0.8413447460685429...
+    one = orc.peer_forward(torch.ones(1, 1, dtype=torch.float64), torch.ones(1, 1, dtype=torch.float64),
+                           torch.ones(1, 1, dtype=torch.float64), torch.ones(1, 1, dtype=torch.float64),
+                           torch.zeros(1, 1, dtype=torch.int64))
+    assert abs(float(one) - 0.8413447460685429) < 1e-15

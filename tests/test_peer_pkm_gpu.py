@@ -1,5 +1,6 @@
-"""PEER and PKM ops against the eager formulas of the reference's tests (tests/test_peer.py:9-24, tests/test_pkm.py:9-20),
-restated here in float64 on the CPU."""
+"""PEER and PKM ops against the oracle's restatement of the eager formulas of the reference's tests
+(tests/test_peer.py:9-24, tests/test_pkm.py:9-20), evaluated in float64 on the CPU; the oracle functions are pinned by the
+plain-C brute force and closed forms in tests/test_oracle_pins.py."""
 import pytest
 import torch
 
@@ -11,12 +12,11 @@ FRO = {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 1e-3}
 
 
 def peer_reference(x, wd, wu, w, idx):
-    s = (x.unsqueeze(1) * wd[idx]).sum(-1)
-    return ((torch.nn.functional.gelu(s) * w).unsqueeze(-1) * wu[idx]).sum(1)
+    return orc.peer_forward(x, wd, wu, w, idx)
 
 
 def pkm_reference(values, w, idx):
-    return (w.unsqueeze(-1) * values[idx]).sum(1)
+    return orc.pkm_forward(values, w, idx)
 
 
 CASES = [(64, 128, 256, 8),            # row schedule
