@@ -39,6 +39,8 @@ SIGNATURES = {
     "fmoe_expert_workspace_bytes_algo": (_sz, [_i64, _int, _i64, _int, _int, _int]),
     "fmoe_expert_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_expert_forward_algo": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _int, _vp]),
+    "fmoe_expert_bucket_workspace_bytes": (_sz, [_i64]),
+    "fmoe_expert_bucket": (_int, [_vp, _i64, _int, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_mlp_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
     "fmoe_mlp_forward": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_block_workspace_bytes": (_sz, [_i64, _int, _int, _int, _i64, _int, _int]),

@@ -47,6 +47,44 @@ def expert_forward(hidden_states, down_weights, up_weights, indices, routing_wei
     return out
 
 
+def expert_bucketing(indices: torch.Tensor, num_experts: int):
+    """Expert-centric grouping of the (token, k) pairs on the GPU (``fmoe_expert_bucket``): returns
+    ``(sorted_token_ids, expert_offsets, sorted_pair_ids, sorted_expert_ids)``, all int32; the first three are what
+    ``_preprocess_expert_centric_indices_pytorch`` of the reference computes with sort / bincount / cumsum
+    (flash_moe/ops/triton/flash_expert.py:528-577).  Pairs of expert ``e`` occupy slots ``[offsets[e], offsets[e+1])`` in
+    ascending flattened position; ids outside ``[0, num_experts)`` are left out, so the three per-slot tensors have
+    ``T*K`` entries of which the first ``offsets[-1]`` are meaningful.  No host synchronisation."""
+    if indices.dim() != 2 or indices.dtype != torch.int64:
+        raise ValueError("indices must be an int64 tensor (num_tokens, num_experts_per_tok)")
+    dev = _C.require_gpu(indices)
+    idx = indices.contiguous()
+    num_tokens, top_k = idx.shape
+    pairs = num_tokens * top_k
+    offsets = torch.empty(num_experts + 1, device=dev, dtype=torch.int32)
+    sorted_pairs, sorted_tokens, sorted_experts = (torch.empty(pairs, device=dev, dtype=torch.int32) for _ in range(3))
+    L = _C.lib()
+    ws_bytes = L.fmoe_expert_bucket_workspace_bytes(num_experts)
+    ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
+    with torch.cuda.device(dev):
+        status = L.fmoe_expert_bucket(_C.ptr(idx), num_tokens, top_k, num_experts, _C.ptr(offsets), _C.ptr(sorted_pairs),
+                                      _C.ptr(sorted_tokens), _C.ptr(sorted_experts), _C.ptr(ws), ws_bytes,
+                                      _C.current_stream(dev))
+    _C.check(status, "flash_expert bucketing")
+    return sorted_tokens, offsets, sorted_pairs, sorted_experts
+
+
+def preprocess_expert_centric_indices(indices: torch.Tensor, routing_weights: torch.Tensor, num_experts: int):
+    """Same return tuple as the reference's ``_preprocess_expert_centric_indices_pytorch(Indices, G, num_experts)``
+    (flash_moe/ops/triton/flash_expert.py:528-577): ``(sorted_token_ids, sorted_G, expert_offsets, max_pairs_per_expert,
+    sorted_pair_ids)``, for callers written against it.  ``max_pairs_per_expert`` is a host integer, so this helper
+    synchronises like the reference does; the library's own forward and backward never need it.  Every id must lie in
+    ``[0, num_experts)`` (the reference's contract)."""
+    sorted_tokens, offsets, sorted_pairs, _ = expert_bucketing(indices, num_experts)
+    sorted_g = routing_weights.reshape(-1)[sorted_pairs.long()]
+    max_pairs = int((offsets[1:] - offsets[:-1]).max().item()) if num_experts > 0 else 0
+    return sorted_tokens, sorted_g, offsets, max_pairs, sorted_pairs
+
+
 def expert_backward(dexperts_states, hidden_states, down_weights, up_weights, indices, routing_weights):
     """Gradients ``(dhidden_states, ddown_weights, dup_weights, drouting_weights)`` of ``expert_forward``
     (``fmoe_expert_backward``; the reference's _flash_expert_backward, flash_moe/ops/triton/flash_expert.py:654-745).

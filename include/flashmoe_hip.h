@@ -129,6 +129,23 @@ int fmoe_expert_forward(const void* x, const void* down, const void* up, const i
                         const void* gates, int64_t num_tokens, int hidden, int64_t num_experts, int top_k,
                         int dtype, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Expert-centric preprocessing on its own.
+ * Replaces _preprocess_expert_centric_indices_pytorch (flash_moe/ops/triton/flash_expert.py:528-577: flatten the pairs,
+ * sort by expert id, bincount + cumsum), on the GPU and without its host synchronisation:
+ *   expert_offsets    [E+1]   int32   out: pairs of expert e occupy slots [offsets[e], offsets[e+1]); offsets[E] = number
+ *                                     of pairs with an id in [0,E) (ids outside belong to no segment)
+ *   sorted_pair_ids   [T*K]   int32   out: flattened position t*K + k of the pair in each slot; inside a segment in
+ *                                     ascending order (the order of a stable sort; torch.sort in the reference is not
+ *                                     stable, so its order there is unspecified); entries from offsets[E] on are not written
+ *   sorted_token_ids  [T*K]   int32   out, optional (NULL to skip): token of each slot, sorted_pair_ids / K
+ *   sorted_expert_ids [T*K]   int32   out, optional: expert id of each slot
+ * workspace: fmoe_expert_bucket_workspace_bytes(E) bytes, 256-byte aligned.  Requires E and T*K below 2^31. */
+size_t fmoe_expert_bucket_workspace_bytes(int64_t num_experts);
+
+int fmoe_expert_bucket(const int64_t* indices, int64_t num_tokens, int top_k, int64_t num_experts, int32_t* expert_offsets,
+                       int32_t* sorted_pair_ids, int32_t* sorted_token_ids, int32_t* sorted_expert_ids, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* Same operation with the schedule chosen by the caller instead of by problem size (fmoe_expert_forward
  * passes FMOE_EXPERT_AUTO).  Both schedules compute the formula above; they differ in how the table rows
  * travel: whole rows per (token, expert) pair, or 128- or 256-byte column slices, each worked through by
