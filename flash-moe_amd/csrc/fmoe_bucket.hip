@@ -93,23 +93,32 @@ __global__ __launch_bounds__(kScanThreads) void bucket_scan_kernel(int32_t* __re
 }
 
 // Pair p of expert e goes to slot cursor[e]++.  tok[slot] = token * tok_scale and exp[slot] = e * exp_scale are what the
-// consumers index with (ids with scale 1, row byte offsets otherwise).  A pair with an id outside [0,E) takes no slot;
-// its entry of `coef_clear` (optional, [num_pairs]) is zeroed so that a later pass over all pairs reads a defined value.
+// consumers index with (ids with scale 1, row byte offsets otherwise).  A pair with an id outside [0,E) belongs to no
+// segment: its entry of `coef_clear` (optional, [num_pairs]) is zeroed so that a later pass over all pairs reads a
+// defined value, and when `tail` is given it zeroes one of the slots after the last segment (offsets[E] + a ticket from
+// the counter `tail`), so that tok and exp are defined over all num_pairs slots.
 __global__ __launch_bounds__(256) void bucket_fill_kernel(const int64_t* __restrict__ indices, int32_t* __restrict__ cursor,
                                                           int32_t* __restrict__ sorted_pairs, uint32_t* __restrict__ tok,
                                                           uint32_t* __restrict__ exp, float* __restrict__ coef_clear,
+                                                          const int32_t* __restrict__ offsets, int32_t* __restrict__ tail,
                                                           int64_t num_pairs, int64_t num_experts, int top_k,
-                                                          uint32_t tok_scale, uint32_t exp_scale) {
+                                                          uint32_t tok_scale, uint32_t exp_scale, int pack_shift) {
     const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= num_pairs) return;
     const int64_t e = indices[p];
     if (e < 0 || e >= num_experts) {
         if (coef_clear != nullptr) coef_clear[p] = 0.0f;
+        if (tail != nullptr) {
+            const int32_t slot = offsets[num_experts] + atomicAdd(tail, 1);
+            if (tok != nullptr) tok[slot] = 0u;
+            if (exp != nullptr) exp[slot] = 0u;
+        }
         return;
     }
     const int32_t slot = atomicAdd(&cursor[e], 1);
     sorted_pairs[slot] = (int32_t)p;
-    if (tok != nullptr) tok[slot] = (uint32_t)(p / top_k) * tok_scale;
+    // pack_shift: the low bits of the id ride in the token word above that bit (token | (e << shift), truncated)
+    if (tok != nullptr) tok[slot] = (uint32_t)(p / top_k) * tok_scale | (pack_shift ? (uint32_t)e << pack_shift : 0u);
     if (exp != nullptr) exp[slot] = (uint32_t)e * exp_scale;
 }
 
@@ -236,7 +245,7 @@ int bucket_histogram(const int64_t* indices, void* workspace, int64_t num_pairs,
 
 int bucket_scan_fill(const int64_t* indices, void* workspace, int64_t num_pairs, int64_t num_experts, int top_k,
                      int32_t* offsets, int32_t* sorted_pairs, uint32_t* tok, uint32_t tok_scale, uint32_t* exp,
-                     uint32_t exp_scale, float* coef_clear, int ordered, hipStream_t stream) {
+                     uint32_t exp_scale, float* coef_clear, int pack_shift, int ordered, hipStream_t stream) {
     const BucketPlan p = plan_bucket(num_experts);
     char* ws = (char*)workspace;
     hipLaunchKernelGGL(bucket_scan_kernel, dim3((unsigned)p.tiles), dim3(kScanThreads), 0, stream, (int32_t*)(ws + p.off_cursor),
@@ -244,8 +253,9 @@ int bucket_scan_fill(const int64_t* indices, void* workspace, int64_t num_pairs,
     FMOE_CHECK_LAUNCH("expert bucketing (scan)");
     if (num_pairs == 0) return FMOE_OK;
     hipLaunchKernelGGL(bucket_fill_kernel, dim3((unsigned)((num_pairs + 255) / 256)), dim3(256), 0, stream, indices,
-                       (int32_t*)(ws + p.off_cursor), sorted_pairs, tok, exp, coef_clear, num_pairs, num_experts, top_k,
-                       tok_scale, exp_scale);
+                       (int32_t*)(ws + p.off_cursor), sorted_pairs, tok, exp, coef_clear, (const int32_t*)offsets,
+                       (tok != nullptr || exp != nullptr) ? (int32_t*)(ws + p.off_ticket) + 1 : nullptr, num_pairs, num_experts,
+                       top_k, tok_scale, exp_scale, pack_shift);
     FMOE_CHECK_LAUNCH("expert bucketing (fill)");
     if (ordered) {
         hipLaunchKernelGGL(bucket_order_kernel, dim3((unsigned)((num_experts + kOrderWaves - 1) / kOrderWaves)),
@@ -283,5 +293,5 @@ extern "C" int fmoe_expert_bucket(const int64_t* indices, int64_t num_tokens, in
         if (int rc = bucket_histogram(indices, workspace, pairs, num_experts, s)) return rc;
     // with no pairs the scan of the cleared counts still writes the all-zero offsets
     return bucket_scan_fill(indices, workspace, pairs, num_experts, top_k > 0 ? top_k : 1, expert_offsets, sorted_pair_ids,
-                            (uint32_t*)sorted_token_ids, 1u, (uint32_t*)sorted_expert_ids, 1u, nullptr, 1, s);
+                            (uint32_t*)sorted_token_ids, 1u, (uint32_t*)sorted_expert_ids, 1u, nullptr, 0, 1, s);
 }

@@ -72,14 +72,15 @@ int expert_slice_states(const float* coef, const void* table, const uint32_t* of
 // (bucket_counts; cleared by bucket_clear, filled by bucket_histogram or by a caller's own kernel) and the scan state.
 // bucket_scan_fill turns the counts into offsets [E+1] and writes, per slot of the grouped order, the pair index, and
 // optionally token * tok_scale and expert * exp_scale; `coef_clear` [num_pairs] gets a zero for every pair whose id is
-// outside [0,E); `ordered` puts every segment in ascending pair index.
+// outside [0,E); with `pack_shift` the token word also carries the id, shifted left by that many bits (truncated to 32
+// bits); `ordered` puts every segment in ascending pair index (and rewrites the token words without packing).
 size_t bucket_workspace_bytes(int64_t num_experts);
 int32_t* bucket_counts(void* workspace);
 int bucket_clear(void* workspace, int64_t num_experts, hipStream_t stream);
 int bucket_histogram(const int64_t* indices, void* workspace, int64_t num_pairs, int64_t num_experts, hipStream_t stream);
 int bucket_scan_fill(const int64_t* indices, void* workspace, int64_t num_pairs, int64_t num_experts, int top_k,
                      int32_t* offsets, int32_t* sorted_pairs, uint32_t* tok, uint32_t tok_scale, uint32_t* exp,
-                     uint32_t exp_scale, float* coef_clear, int ordered, hipStream_t stream);
+                     uint32_t exp_scale, float* coef_clear, int pack_shift, int ordered, hipStream_t stream);
 
 // Plain library GEMM (rocBLAS, loaded on first use) for the operand layouts of the backward passes; row-major
 // C[M,N] = A[M,K] B[K,N] (kBlasNN) or A[K,M]^T B[K,N] (kBlasTN), C = product + beta * C.  Defined in fmoe_mlp_backward.hip.

@@ -8,6 +8,8 @@
 // written once at the end: no atomics, no zero-initialised output, deterministic summation order.
 // Rows of several pairs are requested before any of them is consumed so that enough bytes are in
 // flight to cover HBM / Infinity-Cache latency.
+#include <type_traits>
+
 #include "fmoe_common.h"
 #include "fmoe_vec.h"
 
@@ -31,10 +33,10 @@ constexpr int kWavesPerBlock = 4;
 // waves share one token, wave w taking pairs w*P .. w*P+P-1, (w+4)*P .. of it (P = pairs in flight), and their partial rows
 // are added in wave order through LDS: four times shorter dependency chains when there are not enough tokens to fill the
 // chip with one wave each.
-template <typename T, int NCH, int ACT, bool SPLIT>
+template <typename T, typename TG, int NCH, int ACT, bool SPLIT>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
     const T* __restrict__ x, const T* __restrict__ down, const T* __restrict__ up,
-    const int64_t* __restrict__ indices, const T* __restrict__ gates, T* __restrict__ out,
+    const int64_t* __restrict__ indices, const TG* __restrict__ gates, T* __restrict__ out,
     int64_t num_tokens, int hidden, int64_t num_experts, int top_k) {
     constexpr int V = Elem<T>::kVec;
     const int lane = lane_id();
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
         for (int v = 0; v < V; ++v) acc[c][v] = 0.0f;
 
     const int64_t* my_idx = indices + token * top_k;
-    const T* my_gate = gates + token * top_k;
+    const TG* my_gate = gates + token * top_k;
 
     const int k_first = SPLIT ? wave * kPairsInFlight : 0;
     const int k_step = SPLIT ? kWavesPerBlock * kPairsInFlight : kPairsInFlight;
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void expert_token_kernel(
             gate[u] = 0.0f;
             if (k < top_k) {
                 e = my_idx[k];
-                gate[u] = Elem<T>::to_f32(my_gate[k]);
+                gate[u] = Elem<TG>::to_f32(my_gate[k]);
             }
             // ids are uniform across the wave; make that visible so row addresses live in SGPRs
             const uint32_t elo = __builtin_amdgcn_readfirstlane((uint32_t)(e & 0xffffffff));
@@ -150,10 +152,10 @@ int launch_expert_rows(int act, const void* x, const void* down, const void* up,
 #define FMOE_LAUNCH_EXPERT_ACT(N, A)                                                                                  \
     do {                                                                                                              \
         if (split)                                                                                                    \
-            hipLaunchKernelGGL((expert_token_kernel<T, N, A, true>), grid, block, 0, stream, (const T*)x, (const T*)down, \
+            hipLaunchKernelGGL((expert_token_kernel<T, T, N, A, true>), grid, block, 0, stream, (const T*)x, (const T*)down, \
                                (const T*)up, indices, (const T*)gates, (T*)out, T_, H, E, K);                         \
         else                                                                                                          \
-            hipLaunchKernelGGL((expert_token_kernel<T, N, A, false>), grid, block, 0, stream, (const T*)x, (const T*)down, \
+            hipLaunchKernelGGL((expert_token_kernel<T, T, N, A, false>), grid, block, 0, stream, (const T*)x, (const T*)down, \
                                (const T*)up, indices, (const T*)gates, (T*)out, T_, H, E, K);                         \
     } while (0)
 #define FMOE_LAUNCH_EXPERT(N)                                     \
@@ -174,6 +176,31 @@ int launch_expert_rows(int act, const void* x, const void* down, const void* up,
 #undef FMOE_LAUNCH_EXPERT
 #undef FMOE_LAUNCH_EXPERT_ACT
     FMOE_CHECK_LAUNCH("fmoe_expert_forward");
+    return FMOE_OK;
+}
+
+// out[t] = sum_k coef[t,k] * up[idx[t,k]] with fp32 coefficients that are already complete (the second phase of the
+// bucketed schedule): the row kernel without its score phase.
+template <typename T>
+int launch_expert_rows_coef(const void* up, const int64_t* indices, const float* coef, int64_t T_, int H, int64_t E, int K,
+                            void* out, hipStream_t stream) {
+    constexpr int V = Elem<T>::kVec;
+    const int nch = (H / V + kWave - 1) / kWave;
+    const dim3 block(kWavesPerBlock * kWave);
+    const dim3 grid((unsigned)((T_ + kWavesPerBlock - 1) / kWavesPerBlock));
+#define FMOE_LAUNCH_COEF(N)                                                                                             \
+    hipLaunchKernelGGL((expert_token_kernel<T, float, N, kActNone, false>), grid, block, 0, stream, (const T*)up, (const T*)up, \
+                       (const T*)up, indices, coef, (T*)out, T_, H, E, K)
+    if (nch <= 1) FMOE_LAUNCH_COEF(1);
+    else if (nch <= 2) FMOE_LAUNCH_COEF(2);
+    else if (nch <= 4) FMOE_LAUNCH_COEF(4);
+    else if (nch <= 8) FMOE_LAUNCH_COEF(8);
+    else {
+        set_error("fmoe_expert_forward: hidden=%d exceeds the %d elements per row this build supports", H, 8 * kWave * V);
+        return FMOE_ERR_UNSUPPORTED;
+    }
+#undef FMOE_LAUNCH_COEF
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(states)");
     return FMOE_OK;
 }
 
@@ -209,6 +236,10 @@ __device__ inline __amdgpu_buffer_rsrc_t table_resource(const void* base, uint32
 }
 __device__ inline u32x4_t load_row_piece(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset) {
     return __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0));
+}
+// The same load marked non-temporal: data that is read once and should not displace what the L2 is meant to keep.
+__device__ inline u32x4_t load_row_piece_streaming(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset) {
+    return __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 2));
 }
 
 // ids -> byte offset of the row (kBadOffset if the id is outside [0,E))
@@ -474,12 +505,311 @@ int launch_expert_slices(int act, const void* x, const void* down, const void* u
     return launch_expert_slices_prepared<T>(act, x, down, up, gates, T_, H, E, K, out, workspace, stream);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Bucketed (expert-centric) schedule, for tables too large for the column-slice schedule.
+//
+// The pairs are grouped by expert (fmoe_bucket.hip).  In that order consecutive pairs share their row of `down`, so a
+// lane group keeps the row's piece in registers and only the pieces of x are gathered, one per pair; and it is x, not
+// the table, that has to stay in L2: column bands of x (128 to 512 bytes per token, at most about 4 MiB for all tokens)
+// are dealt to the XCDs like the slices above, while every table byte streams through once, in order.
+//   bucket  : ids -> offsets[E+1], per slot of the grouped order: pair index, x row offset, table row offset
+//   scores  : spart[band][slot] = <x[token, band cols], down[expert, band cols]>
+//   gate    : a[pair] = act(sum_band spart[band][slot]) * gate[pair]        (back in (token, k) order)
+//   states  : out[token] = sum_k a[token,k] * up[expert_k]                  (one wave per token, whole rows)
+// ------------------------------------------------------------------------------------------------
+constexpr int kBucketChunk = 64;     // consecutive slots one lane group works through
+constexpr int kBucketBatch = 8;      // slots whose loads are in flight together
+
+// xb[band][token][band bytes] = x[token][band * band bytes ...]: every band of x contiguous.  Pieces of one band that
+// lie a whole row (a power of two, typically) apart compete for a few sets of the L2; contiguous, the band uses them all.
+__global__ __launch_bounds__(256) void expert_band_copy_kernel(const u32x4_t* __restrict__ x, u32x4_t* __restrict__ xb,
+                                                               int64_t num_tokens, int row_packets, int band_packets) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;       // packet index in x
+    if (i >= num_tokens * row_packets) return;
+    const int64_t t = i / row_packets;
+    const int pk = (int)(i % row_packets), band = pk / band_packets, c = pk % band_packets;
+    xb[((int64_t)band * num_tokens + t) * band_packets + c] = x[i];
+}
+
+// CL lanes share one pair: a band is CL * 16 bytes wide and a wave-wide load covers G = 64 / CL pairs.  A workgroup
+// takes runs of 4 * G * kBucketChunk consecutive slots; each of its 4 * G lane groups works through kBucketChunk of them,
+// kBucketBatch at a time.  The experts of such a run are consecutive rows of the table: their pieces of the band are
+// staged in LDS with plain coalesced loads (every byte of the band leaves the table once; the loads are issued one run
+// ahead and parked in registers), and a slot reads its piece from there, so that the only vector-memory instruction
+// per slot is the gather of x: the kernel is bound by the rate at which a CU takes 64-lane loads (about 30 cycles
+// each), not by bytes.  A run whose experts span more rows than fit (few pairs for many experts) loads the pieces per
+// slot instead.
+// entry[slot] = token | (expert & 255) << 24: with at most 256 staged rows the low byte of the id places the row.
+constexpr int kBucketLdsBytes = 32768;     // staged rows per workgroup: 32 KiB / band width, at most 256
+constexpr uint32_t kEntryTokenMask = 0x00FFFFFFu;
+
+template <typename T, int CL>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void expert_scores_bucketed_kernel(
+    const T* __restrict__ xb, uint32_t x_bytes, const T* __restrict__ down, uint32_t table_bytes,
+    const uint32_t* __restrict__ entry, const uint32_t* __restrict__ expid, const int32_t* __restrict__ offsets,
+    int64_t num_experts, float* __restrict__ spart, int64_t spart_stride, uint32_t row_bytes, int num_bands, int parts,
+    int blocks_per_unit) {
+    constexpr int G = kWave / CL, U = kBucketBatch;
+    constexpr int kRun = 4 * G * kBucketChunk;                          // slots per workgroup iteration
+    constexpr int kBand = CL * 16;
+    constexpr int kRows = kBucketLdsBytes / kBand;
+    constexpr int kStage = kBucketLdsBytes / 16 / 256;                  // 16-byte pieces per thread that fill the LDS
+    static_assert(kBucketChunk == 8 * U && CL >= 8 && kRows <= 256, "lane c < 8 holds the entries of batch c");
+    __shared__ __attribute__((aligned(16))) unsigned char rows[kBucketLdsBytes];
+    const int b = (int)blockIdx.x;
+    const int unit = (b & 7) + 8 * ((b >> 3) / blocks_per_unit);       // XCD (b & 7) takes units x, x + 8, ...
+    const int tb = (b >> 3) % blocks_per_unit;
+    if (unit >= num_bands * parts) return;
+    const int band = unit % num_bands, part = unit / num_bands;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & (CL - 1), g = lane / CL;
+    const int group_base = (lane & ~(CL - 1)) << 2;                     // byte address of the group's lane 0 for ds_bpermute
+    const uint32_t col_bytes = (uint32_t)band * kBand + (uint32_t)c * 16;
+    const uint32_t x_col_bytes = (uint32_t)band * (x_bytes / (uint32_t)num_bands) + (uint32_t)c * 16;   // x is band-major here
+    const __amdgpu_buffer_rsrc_t xr = table_resource(xb, x_bytes), wr = table_resource(down, table_bytes);
+    const __amdgpu_buffer_rsrc_t er = table_resource(entry, (uint32_t)spart_stride * 4u);
+    const int n_valid = offsets[num_experts];
+    const int runs = (n_valid + kRun - 1) / kRun;
+    const int per_part = (runs + parts - 1) / parts;
+    const int run_end = (part + 1) * per_part < runs ? (part + 1) * per_part : runs;
+    float* my_spart = spart + (int64_t)band * spart_stride;
+
+    // entries of the group's 64 slots: lanes 0..7 of the group hold 8 each (reads past the array give zeros; slots from
+    // n_valid on are not stored)
+    auto load_entries = [&](int run, u32x4_t (&t)[2]) {
+        const uint32_t at = ((uint32_t)run * kRun + (uint32_t)(wave * G + g) * kBucketChunk + (uint32_t)(c & 7) * 8u) * 4u;
+        t[0] = load_row_piece_streaming(er, at);
+        t[1] = load_row_piece_streaming(er, at + 16u);
+    };
+    // first and last expert of a run (the slots are in ascending expert order)
+    auto load_span = [&](int run, uint32_t& lo, uint32_t& hi) {
+        const int q_lo = run * kRun, q_hi = (run + 1) * kRun < n_valid ? (run + 1) * kRun - 1 : n_valid - 1;
+        lo = expid[q_lo];
+        hi = expid[q_hi];
+    };
+    // piece k of thread i: row (i + 256 k) / CL of the run, packet (i + 256 k) % CL of the band
+    auto load_rows = [&](uint32_t lo, uint32_t hi, u32x4_t (&st)[kStage]) {
+        const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)lo);
+        const uint32_t span = (uint32_t)__builtin_amdgcn_readfirstlane((int)hi) - first + 1u;
+        if (span > (uint32_t)kRows) return;
+#pragma unroll
+        for (int k = 0; k < kStage; ++k) {
+            const uint32_t i = (uint32_t)tid + 256u * k, r = i / CL;
+            st[k] = load_row_piece_streaming(wr, r < span ? (first + r) * row_bytes + (uint32_t)band * kBand + (i % CL) * 16u : kBadOffset);
+        }
+    };
+    int run = part * per_part + tb;
+    u32x4_t ent[2], stage[kStage];
+    uint32_t e_lo = 0, e_hi = 0, n_lo = 0, n_hi = 0;                    // expert span of this run and of the next one
+    if (run < run_end) {
+        load_entries(run, ent);
+        load_span(run, e_lo, e_hi);
+        load_span(run + blocks_per_unit < run_end ? run + blocks_per_unit : run, n_lo, n_hi);
+        load_rows(e_lo, e_hi, stage);
+    }
+    for (; run < run_end; run += blocks_per_unit) {
+        const int next = run + blocks_per_unit < run_end ? run + blocks_per_unit : run;
+        const int next2 = next + blocks_per_unit < run_end ? next + blocks_per_unit : next;
+        const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)e_lo);
+        const uint32_t span = (uint32_t)__builtin_amdgcn_readfirstlane((int)e_hi) - first + 1u;
+        const bool staged = span <= (uint32_t)kRows;
+        if (staged) {
+#pragma unroll
+            for (int k = 0; k < kStage; ++k)
+                *reinterpret_cast<u32x4_t*>(&rows[((uint32_t)tid + 256u * k) * 16u]) = stage[k];
+        }
+        __syncthreads();
+        u32x4_t nxt[2];
+        uint32_t f_lo, f_hi;
+        load_entries(next, nxt);                                        // the next run's entries and rows, ahead of time
+        load_span(next2, f_lo, f_hi);
+        load_rows(n_lo, n_hi, stage);
+        const int q_first = run * kRun + (wave * G + g) * kBucketChunk;
+        if (staged) {
+            const uint32_t lds_base = (uint32_t)c * 16u - (first & 255u) * kBand;     // + (entry >> 24) * kBand, modulo the LDS size
+#pragma unroll 1
+            for (int bt = 0; bt < kBucketChunk / U; ++bt) {
+                const int q0 = q_first + bt * U;
+                if (q0 >= n_valid) break;
+                const int src = group_base + bt * 4;                    // lane bt of the group holds this batch's entries
+                u32x4_t xg[U];
+                uint32_t at[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t en = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)ent[u / 4][u % 4]);
+                    xg[u] = load_row_piece(xr, (en & kEntryTokenMask) * kBand + x_col_bytes);
+                    at[u] = ((en >> 24) * kBand + lds_base) & (uint32_t)(kBucketLdsBytes - 1);
+                }
+                float partial[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    partial[u] = dot16<T>(xg[u], *reinterpret_cast<const u32x4_t*>(&rows[at[u]]), 0.0f);
+                float total = transpose_sum<U, 1>(partial, c);          // over each aligned 8 lanes: slot q0 + (c & 7)
+                if constexpr (CL >= 16) total += xor_step<U, 8>(total);
+                if constexpr (CL >= 32) total += xor_step<U, 16>(total);
+                if (c < U && q0 + c < n_valid) __builtin_nontemporal_store(total, &my_spart[q0 + c]);
+            }
+        } else {
+            // the experts of this run are too far apart to stage: each slot loads its own piece of the row
+#pragma unroll 1
+            for (int bt = 0; bt < kBucketChunk / U; ++bt) {
+                const int q0 = q_first + bt * U;
+                if (q0 >= n_valid) break;
+                const int src = group_base + bt * 4;
+                float partial[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t en = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)ent[u / 4][u % 4]);
+                    const uint32_t e = q0 + u < n_valid ? expid[q0 + u] : 0u;
+                    const u32x4_t xg = load_row_piece(xr, (en & kEntryTokenMask) * kBand + x_col_bytes);
+                    partial[u] = dot16<T>(xg, load_row_piece(wr, e * row_bytes + col_bytes), 0.0f);
+                }
+                float total = transpose_sum<U, 1>(partial, c);
+                if constexpr (CL >= 16) total += xor_step<U, 8>(total);
+                if constexpr (CL >= 32) total += xor_step<U, 16>(total);
+                if (c < U && q0 + c < n_valid) __builtin_nontemporal_store(total, &my_spart[q0 + c]);
+            }
+        }
+        __syncthreads();                                                // the rows are rewritten by the next run
+        ent[0] = nxt[0];
+        ent[1] = nxt[1];
+        e_lo = n_lo;
+        e_hi = n_hi;
+        n_lo = f_lo;
+        n_hi = f_hi;
+    }
+}
+
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void expert_gate_sorted_kernel(const float* __restrict__ spart, int64_t spart_stride,
+                                                                 const T* __restrict__ gates, const int32_t* __restrict__ sorted_pairs,
+                                                                 const int32_t* __restrict__ offsets, int64_t num_experts,
+                                                                 float* __restrict__ a, int num_bands) {
+    const int n_valid = offsets[num_experts];
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < n_valid; q += (int64_t)gridDim.x * blockDim.x) {
+        const int32_t p = sorted_pairs[q];
+        const float gate = Elem<T>::to_f32(gates[p]);
+        float s = 0.0f;
+        int bd = 0;
+        for (; bd + 8 <= num_bands; bd += 8) {              // eight loads in flight at a time, summed in band order
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_nontemporal_load(&spart[(int64_t)(bd + j) * spart_stride + q]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s += v[j];
+        }
+        for (; bd < num_bands; ++bd) s += spart[(int64_t)bd * spart_stride + q];
+        a[p] = activate<ACT>(s) * gate;
+    }
+}
+
+struct BucketedPlan {
+    int chunk_lanes, num_bands, parts, blocks_per_unit;
+    unsigned grid;
+    size_t off_bucket, off_offsets, off_pairs, off_tok, off_exp, off_a, off_spart, off_xb, bytes;
+};
+
+// Band width: as wide as lets the band of all tokens stay in one XCD's L2 (about 2 MiB of its 4), at least 128 bytes.
+BucketedPlan plan_bucketed(int64_t T_, int H, int64_t E, int K, size_t elt) {
+    BucketedPlan p;
+    p.chunk_lanes = T_ * 512 <= (2ll << 20) ? 32 : (T_ * 256 <= (2ll << 20) ? 16 : 8);
+    while (p.chunk_lanes > 8 && (H * elt) % ((size_t)p.chunk_lanes * 16) != 0) p.chunk_lanes /= 2;   // bands tile the row
+    const size_t band_bytes = (size_t)p.chunk_lanes * 16;
+    p.num_bands = (int)((H * elt + band_bytes - 1) / band_bytes);
+    p.parts = (p.num_bands < 8 && 8 % p.num_bands == 0) ? 8 / p.num_bands : 1;      // several XCDs share a band
+    const int64_t pairs = T_ * K;
+    const int64_t run_slots = 4 * (kWave / p.chunk_lanes) * kBucketChunk;
+    const int64_t want = ((pairs + run_slots - 1) / run_slots + p.parts - 1) / p.parts;      // runs per part
+    p.blocks_per_unit = (int)(want < 1 ? 1 : (want > 256 ? 256 : want));
+    const int units = p.num_bands * p.parts;
+    p.grid = (unsigned)(8 * p.blocks_per_unit * ((units + 7) / 8));
+    size_t o = 0;
+    auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
+    p.off_bucket = take(bucket_workspace_bytes(E));
+    p.off_offsets = take((size_t)(E + 1) * 4);
+    p.off_pairs = take((size_t)pairs * 4);
+    p.off_tok = take((size_t)pairs * 4);
+    p.off_exp = take((size_t)pairs * 4);
+    p.off_a = take((size_t)pairs * 4);
+    p.off_spart = take((size_t)p.num_bands * pairs * 4);
+    p.off_xb = take((size_t)T_ * H * elt);
+    p.bytes = o;
+    return p;
+}
+
+bool bucketed_possible(int64_t T_, int64_t E, int H, int K, size_t elt) {
+    return (H * elt) % 128 == 0 &&      // whole 128-byte bands
+           (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset && (uint64_t)T_ * (uint64_t)H * elt < (uint64_t)kBadOffset &&
+           T_ * (int64_t)K < (1ll << 31) - 4096 && E < (1ll << 31) - 1 && T_ <= (int64_t)kEntryTokenMask;
+}
+
+template <typename T>
+int launch_expert_bucketed(int act, const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
+                           int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+    const BucketedPlan p = plan_bucketed(T_, H, E, K, sizeof(T));
+    char* ws = (char*)workspace;
+    int32_t* offsets = (int32_t*)(ws + p.off_offsets);
+    int32_t* sorted_pairs = (int32_t*)(ws + p.off_pairs);
+    uint32_t* tokoff = (uint32_t*)(ws + p.off_tok);
+    uint32_t* expoff = (uint32_t*)(ws + p.off_exp);
+    float* a = (float*)(ws + p.off_a);
+    float* spart = (float*)(ws + p.off_spart);
+    const int64_t pairs = T_ * K;
+    const uint32_t row_bytes = (uint32_t)(H * sizeof(T));
+    if (act == kActNone) {
+        // no score phase: the coefficient is the routing weight itself, nothing to group
+        return launch_expert_rows<T>(act, x, down, up, indices, gates, T_, H, E, K, out, stream);
+    }
+    if (int rc = bucket_clear(ws + p.off_bucket, E, stream)) return rc;
+    if (int rc = bucket_histogram(indices, ws + p.off_bucket, pairs, E, stream)) return rc;
+    if (int rc = bucket_scan_fill(indices, ws + p.off_bucket, pairs, E, K, offsets, sorted_pairs, tokoff, 1u, expoff, 1u, a, 24,
+                                  0, stream))
+        return rc;
+    void* xb = ws + p.off_xb;
+    {
+        const int64_t packets = T_ * (int64_t)(row_bytes / 16);
+        hipLaunchKernelGGL(expert_band_copy_kernel, dim3((unsigned)((packets + 255) / 256)), dim3(256), 0, stream,
+                           (const u32x4_t*)x, (u32x4_t*)xb, T_, (int)(row_bytes / 16), p.chunk_lanes);
+        FMOE_CHECK_LAUNCH("fmoe_expert_forward(band copy)");
+    }
+    const uint32_t x_bytes = (uint32_t)(T_ * (int64_t)row_bytes), table_bytes = (uint32_t)(E * (int64_t)row_bytes);
+#define FMOE_LAUNCH_BUCKETED(CLV)                                                                                          \
+    hipLaunchKernelGGL((expert_scores_bucketed_kernel<T, CLV>), dim3(p.grid), dim3(256), 0, stream, (const T*)xb, x_bytes,  \
+                       (const T*)down, table_bytes, (const uint32_t*)tokoff, (const uint32_t*)expoff, (const int32_t*)offsets, \
+                       E, spart, pairs, row_bytes, p.num_bands, p.parts, p.blocks_per_unit)
+    if (p.chunk_lanes == 32) FMOE_LAUNCH_BUCKETED(32);
+    else if (p.chunk_lanes == 16) FMOE_LAUNCH_BUCKETED(16);
+    else FMOE_LAUNCH_BUCKETED(8);
+#undef FMOE_LAUNCH_BUCKETED
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(bucketed scores)");
+    const unsigned flat_grid = (unsigned)((pairs + 255) / 256 < 16384 ? (pairs + 255) / 256 : 16384);
+    if (act == kActSilu)
+        hipLaunchKernelGGL((expert_gate_sorted_kernel<T, kActSilu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
+                           pairs, (const T*)gates, (const int32_t*)sorted_pairs, (const int32_t*)offsets, E, a, p.num_bands);
+    else
+        hipLaunchKernelGGL((expert_gate_sorted_kernel<T, kActGelu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
+                           pairs, (const T*)gates, (const int32_t*)sorted_pairs, (const int32_t*)offsets, E, a, p.num_bands);
+    FMOE_CHECK_LAUNCH("fmoe_expert_forward(bucketed gate)");
+    return launch_expert_rows_coef<T>(up, indices, a, T_, H, E, K, out, stream);
+}
+
 // A slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic; with 128-byte
 // slices of up to 8 MiB the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
 // too few pairs to pay for four launches, whole rows are gathered by the one-wave-per-token kernel.
 bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) && T_ * K >= (1ll << 16); }
 // rows are addressed with 32-bit byte offsets below kBadOffset
 bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
+
+// Which schedule a call takes.  A forced schedule that cannot run these extents is reported by the dispatcher; AUTO
+// falls back to whole rows.
+bool buckets_pay(int64_t T_, int64_t E, int K) { return !slices_pay(T_, E, K) && T_ * K >= (1ll << 16); }
+int choose_schedule(int algo, int64_t T_, int H, int64_t E, int K, size_t elt) {
+    if (K == 0) return FMOE_EXPERT_ROWS;
+    if (algo != FMOE_EXPERT_AUTO) return algo;
+    if (slices_pay(T_, E, K) && slices_possible(E, H, elt)) return FMOE_EXPERT_SLICES;
+    if (buckets_pay(T_, E, K) && bucketed_possible(T_, E, H, K, elt)) return FMOE_EXPERT_BUCKETS;
+    return FMOE_EXPERT_ROWS;
+}
 
 }  // namespace
 
@@ -536,9 +866,12 @@ extern "C" size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidde
                                                    int algo) {
     using namespace fmoe;
     if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0 || top_k <= 0 || !dtype_ok(dtype)) return 0;
-    const bool possible = slices_possible(num_experts, hidden, dtype_size(dtype));
-    const bool slices = algo == FMOE_EXPERT_SLICES || (algo == FMOE_EXPERT_AUTO && possible && slices_pay(num_tokens, num_experts, top_k));
-    return slices ? plan_slices(num_tokens, hidden, num_experts, top_k, dtype_size(dtype)).bytes : 0;   // the row schedule needs no scratch
+    const size_t elt = dtype_size(dtype);
+    switch (choose_schedule(algo, num_tokens, hidden, num_experts, top_k, elt)) {
+        case FMOE_EXPERT_SLICES: return plan_slices(num_tokens, hidden, num_experts, top_k, elt).bytes;
+        case FMOE_EXPERT_BUCKETS: return plan_bucketed(num_tokens, hidden, num_experts, top_k, elt).bytes;
+        default: return 0;   // the row schedule needs no scratch
+    }
 }
 
 extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
@@ -557,7 +890,7 @@ int expert_dispatch(const char* who, int act, const void* x, const void* down, c
     FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_experts > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
                  "%s: bad shape T=%lld H=%d E=%lld K=%d", who, (long long)num_tokens, hidden,
                  (long long)num_experts, top_k);
-    FMOE_REQUIRE(algo >= FMOE_EXPERT_AUTO && algo <= FMOE_EXPERT_SLICES, FMOE_ERR_UNSUPPORTED,
+    FMOE_REQUIRE(algo >= FMOE_EXPERT_AUTO && algo <= FMOE_EXPERT_BUCKETS, FMOE_ERR_UNSUPPORTED,
                  "%s: unknown algo %d", who, algo);
     if (num_tokens == 0) return FMOE_OK;
     FMOE_REQUIRE((x || act == kActNone) && (down || act == kActNone) && up && out, FMOE_ERR_NULL_POINTER, "%s: null tensor pointer", who);
@@ -572,14 +905,23 @@ int expert_dispatch(const char* who, int act, const void* x, const void* down, c
                  "%s: problem too large (E=%lld, pairs=%lld)", who, (long long)num_experts,
                  (long long)(num_tokens * top_k));
     hipStream_t s = (hipStream_t)stream;
-    bool slices = algo == FMOE_EXPERT_SLICES || (algo == FMOE_EXPERT_AUTO && slices_pay(num_tokens, num_experts, top_k));
-    if (top_k == 0) slices = false;
-    if (slices && !slices_possible(num_experts, hidden, dtype_size(dtype))) {
-        FMOE_REQUIRE(algo == FMOE_EXPERT_AUTO, FMOE_ERR_UNSUPPORTED,
-                     "%s: tables of 4 GiB or more cannot use the column-slice schedule", who);
-        slices = false;
+    const size_t elt = dtype_size(dtype);
+    const int schedule = choose_schedule(algo, num_tokens, hidden, num_experts, top_k, elt);
+    FMOE_REQUIRE(schedule != FMOE_EXPERT_SLICES || slices_possible(num_experts, hidden, elt), FMOE_ERR_UNSUPPORTED,
+                 "%s: tables of 4 GiB or more cannot use the column-slice schedule", who);
+    FMOE_REQUIRE(schedule != FMOE_EXPERT_BUCKETS || bucketed_possible(num_tokens, num_experts, hidden, top_k, elt),
+                 FMOE_ERR_UNSUPPORTED, "%s: the bucketed schedule needs rows that are multiples of 128 bytes, x and each table below 4 GiB and fewer than 2^31 pairs", who);
+    if (schedule == FMOE_EXPERT_BUCKETS) {
+        const size_t need = fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, dtype, FMOE_EXPERT_BUCKETS);
+        FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
+                     "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+        switch (dtype) {
+            case FMOE_F32: return launch_expert_bucketed<float>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            case FMOE_BF16: return launch_expert_bucketed<bf16_t>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+            default: return launch_expert_bucketed<f16_t>(act, x, down, up, indices, gates, num_tokens, hidden, num_experts, top_k, out, workspace, s);
+        }
     }
-    if (slices) {
+    if (schedule == FMOE_EXPERT_SLICES) {
         const size_t need = fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, dtype, FMOE_EXPERT_SLICES);
         FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
                      "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);

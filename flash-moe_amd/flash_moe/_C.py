@@ -21,7 +21,7 @@ _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 
 ERR_TOPK_RANGE = -3
 
-EXPERT_AUTO, EXPERT_ROWS, EXPERT_SLICES = 0, 1, 2
+EXPERT_AUTO, EXPERT_ROWS, EXPERT_SLICES, EXPERT_BUCKETS = 0, 1, 2, 3
 
 _vp, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
 

@@ -147,14 +147,17 @@ int fmoe_expert_bucket(const int64_t* indices, int64_t num_tokens, int top_k, in
                        size_t workspace_bytes, void* stream);
 
 /* Same operation with the schedule chosen by the caller instead of by problem size (fmoe_expert_forward
- * passes FMOE_EXPERT_AUTO).  Both schedules compute the formula above; they differ in how the table rows
- * travel: whole rows per (token, expert) pair, or 128- or 256-byte column slices, each worked through by
- * one XCD (one L2) at a time.
+ * passes FMOE_EXPERT_AUTO).  All schedules compute the formula above; they differ in how the table rows
+ * travel: whole rows per (token, expert) pair; 128- or 256-byte column slices of the tables, each worked through by
+ * one XCD (one L2) at a time; or, for tables far larger than the L2s, pairs grouped by expert so that the scores
+ * stream each down row once against column bands of x.
  * The reference has one schedule (expert-centric Triton kernels, flash_expert.py:580-651). */
 typedef enum {
     FMOE_EXPERT_AUTO = 0,
     FMOE_EXPERT_ROWS = 1,     /* one wavefront per token, whole rows; no workspace needed */
-    FMOE_EXPERT_SLICES = 2    /* column slices resident in L2; needs the workspace */
+    FMOE_EXPERT_SLICES = 2,   /* column slices of the tables resident in L2; needs the workspace */
+    FMOE_EXPERT_BUCKETS = 3   /* pairs grouped by expert (the fmoe_expert_bucket stage), column bands of x resident in
+                                 L2, each down row streamed once; needs the workspace */
 } fmoe_expert_algo_t;
 
 int fmoe_expert_forward_algo(const void* x, const void* down, const void* up, const int64_t* indices,

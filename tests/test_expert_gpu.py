@@ -8,7 +8,8 @@ from oracle import flashmoe_oracle as orc
 pytestmark = pytest.mark.gpu
 
 
-ALGOS = {"auto": 0, "rows": 1, "slices": 2}
+ALGOS = {"auto": 0, "rows": 1, "slices": 2, "buckets": 3}
+SCHEDULES = ["rows", "slices", "buckets"]
 
 
 def run(x, wd, wu, idx, g, algo="auto"):
@@ -22,7 +23,7 @@ def truth64(x, wd, wu, idx, g):
     return orc.expert_forward(x.double(), wd.double(), wu.double(), idx, g.double())
 
 
-@pytest.mark.parametrize("algo", ["rows", "slices"])
+@pytest.mark.parametrize("algo", SCHEDULES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,K", [
     (512, 256, 1024, 16),        # C1
@@ -36,6 +37,11 @@ def truth64(x, wd, wu, idx, g):
 def test_expert_matches_oracle(dtype, T, H, E, K, algo):
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=T + K)
     x, wd, wu, g = (t.to(dtype) for t in (x, wd, wu, g))
+    if algo == "buckets" and (H * x.element_size()) % 128 != 0:
+        # the bucketed schedule works on whole 128-byte column bands: forcing it on other rows is refused
+        with pytest.raises(ValueError, match="bucketed schedule"):
+            run(x, wd, wu, idx, g, algo)
+        return
     got = run(x, wd, wu, idx, g, algo)
     assert got.dtype == dtype and got.shape == (T, H)
     # (1) the stated bar: against the oracle run in the same dtype
@@ -45,7 +51,7 @@ def test_expert_matches_oracle(dtype, T, H, E, K, algo):
     assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 5e-4}[dtype], fro
 
 
-@pytest.mark.parametrize("algo", ["rows", "slices"])
+@pytest.mark.parametrize("algo", SCHEDULES)
 def test_expert_reference_test_distribution(algo):
     # distributions of the reference's expert benchmark (tests/test_expert.py:160-175): x ~ N(0,0.5),
     # tables ~ N(0,0.1), ids drawn WITH replacement, gates ~ N(0,0.1) (negative values allowed)
@@ -60,7 +66,7 @@ def test_expert_reference_test_distribution(algo):
     assert rel_fro(got, truth64(x, wd, wu, idx, g)) < 4e-3
 
 
-@pytest.mark.parametrize("algo", ["rows", "slices"])
+@pytest.mark.parametrize("algo", SCHEDULES)
 def test_expert_properties_full_size(algo):
     # C3 at full size: size-independent properties instead of a CPU evaluation of all 1M pairs
     import functools
@@ -91,16 +97,35 @@ def test_expert_properties_full_size(algo):
 
 
 def test_expert_schedules_agree():
-    # the two schedules on the same inputs: same pairs, different summation order (and, for bf16, the
+    # the schedules on the same inputs: same pairs, different summation order (and, for bf16, the
     # slice schedule rounds silu(s)*g to bf16 before the packed dot product)
     T, H, E, K = 2048, 1024, 16384, 64
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=9)
     for dtype, tol in ((torch.float32, 2e-6), (torch.bfloat16, 5e-3)):
         args = tuple(t.to(dtype) if t.is_floating_point() else t for t in (x, wd, wu, idx, g))
-        assert rel_fro(run(*args, algo="slices"), run(*args, algo="rows")) < tol
+        rows = run(*args, algo="rows")
+        assert rel_fro(run(*args, algo="slices"), rows) < tol
+        assert rel_fro(run(*args, algo="buckets"), rows) < tol
 
 
-@pytest.mark.parametrize("algo", ["rows", "slices"])
+def test_expert_large_table_takes_the_bucketed_schedule():
+    """A table far beyond what the column-slice schedule keeps in L2 (C5's expert count and top-k, fewer tokens and a
+    narrower hidden size): the default schedule is the bucketed one, checked against the oracle and the row schedule."""
+    from flash_moe import _C
+
+    T, H, E, K = 1024, 256, 262144, 128
+    assert _C.lib().fmoe_expert_workspace_bytes(T, H, E, K, _C.BF16) == _C.lib().fmoe_expert_workspace_bytes_algo(
+        T, H, E, K, _C.BF16, _C.EXPERT_BUCKETS) > 0
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=21)
+    x, wd, wu, g = (t.bfloat16() for t in (x, wd, wu, g))
+    got = run(x, wd, wu, idx, g, "auto")
+    assert torch.equal(got, run(x, wd, wu, idx, g, "buckets"))
+    assert_output_close(got, orc.expert_forward(x, wd, wu, idx, g), torch.bfloat16, "bucketed schedule vs oracle")
+    assert rel_fro(got, truth64(x, wd, wu, idx, g)) < 4e-3
+    assert rel_fro(got, run(x, wd, wu, idx, g, "rows")) < 4e-3
+
+
+@pytest.mark.parametrize("algo", SCHEDULES)
 def test_expert_duplicates_and_single_expert(algo):
     T, H, E = 64, 256, 32
     x, wd, wu, _, _ = orc.make_expert_inputs(T, H, E, 4, seed=5, std=0.2)
@@ -112,7 +137,7 @@ def test_expert_duplicates_and_single_expert(algo):
     torch.testing.assert_close(one, (torch.nn.functional.silu(s)).unsqueeze(-1) * wu[7], rtol=1e-4, atol=1e-6)
 
 
-@pytest.mark.parametrize("algo", ["rows", "slices"])
+@pytest.mark.parametrize("algo", SCHEDULES)
 def test_expert_out_of_range_ids_contribute_nothing(algo):
     T, H, E, K = 32, 64, 16, 4
     x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=6, std=0.2)
