@@ -358,6 +358,21 @@ template <> __device__ inline void axpy16_pair<bf16_t>(float a0, float a1, u32x4
     }
 }
 
+// acc[0..8) += a * w for one 16-byte packet of a 16-bit row.  bf16: the coefficient is rounded to bf16 (the reference
+// forms silu(s)*g in the activation dtype as well, flash_expert.py:191) and meets each element through the packed dot
+// product, (w[2i], w[2i+1]) . (a, 0) and . (0, a): no unpacking, half the instructions of convert + fma.
+template <typename T> __device__ inline void axpy16_coef(float a, u32x4_t w, float* acc) { axpy16<T>(a, w, acc); }
+template <> __device__ inline void axpy16_coef<bf16_t>(float a, u32x4_t w, float* acc) {
+    const bf16_t ab = (bf16_t)a, zero = (bf16_t)0.0f;
+    const bf16x2_t lo = {ab, zero}, hi = {zero, ab};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t wi = w[i];
+        acc[2 * i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wi), lo, acc[2 * i], false);
+        acc[2 * i + 1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wi), hi, acc[2 * i + 1], false);
+    }
+}
+
 template <typename T, int CL>
 __global__ __launch_bounds__(256) void expert_states_slice_kernel(
     const float* __restrict__ a, const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ off32,
@@ -703,11 +718,191 @@ __global__ __launch_bounds__(256) void expert_gate_sorted_kernel(const float* __
     }
 }
 
+// ---- second phase for large tables: a sweep over the experts with the output in LDS ----------------------------------
+// out[t] = sum_k a[t,k] * up[e_k] needs one row of `up` per pair.  Token by token these rows come from all over a table
+// far larger than the caches (the row schedule: bound by HBM).  Here every lane group owns kSweepTokens tokens and walks
+// their pairs in ascending expert order; all lane groups of an XCD do so at the same pace on the same column band, so at
+// any moment they gather from one narrow window of the band, which the L2 holds: the band leaves HBM once per pass over
+// it.  The running sums of a workgroup's 512 tokens (64 fp32 columns each) live in LDS; a lane group is the only one to
+// touch its tokens' rows, in list order, so the result is deterministic without atomics.
+//   owner sort : per owner (kSweepTokens consecutive tokens) the keys expert << 10 | token_in_owner << 8 | k, sorted,
+//                and the coefficients in that order
+//   sweep      : out[token, band] for 512 tokens x one 128-byte band per workgroup
+constexpr int kSweepTokens = 4;                          // tokens per lane group
+constexpr int kSweepThreads = 1024;                      // 16 waves = 128 lane groups = 512 tokens per workgroup
+constexpr int kSweepWgTokens = (kSweepThreads / 8) * kSweepTokens;
+constexpr int kSweepMaxTopK = 256, kSweepMaxKeys = kSweepTokens * kSweepMaxTopK;
+
+__global__ __launch_bounds__(256) void expert_owner_sort_kernel(const int64_t* __restrict__ indices, const float* __restrict__ a,
+                                                                uint32_t* __restrict__ entries, float* __restrict__ coef,
+                                                                int64_t num_tokens, int64_t num_experts, int top_k) {
+    __shared__ uint32_t keys[kSweepMaxKeys];
+    const int tid = (int)threadIdx.x;
+    const int64_t owner = blockIdx.x;
+    const int n = kSweepTokens * top_k;
+    int m = 64;
+    while (m < n) m <<= 1;
+    for (int i = tid; i < m; i += 256) {
+        uint32_t key = 0xFFFFFFFFu;
+        if (i < n) {
+            const int tl = i / top_k, k = i % top_k;
+            const int64_t t = owner * kSweepTokens + tl;
+            if (t < num_tokens) {
+                const int64_t e = indices[t * top_k + k];
+                if (e >= 0 && e < num_experts) key = (uint32_t)e << 10 | (uint32_t)tl << 8 | (uint32_t)k;
+            }
+        }
+        keys[i] = key;
+    }
+    __syncthreads();
+    for (int k = 2; k <= m; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = tid; i < m / 2; i += 256) {
+                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1)), hi = lo | j;
+                const uint32_t x0 = keys[lo], x1 = keys[hi];
+                if ((x0 > x1) == ((lo & k) == 0)) {
+                    keys[lo] = x1;
+                    keys[hi] = x0;
+                }
+            }
+            __syncthreads();
+        }
+    for (int i = tid; i < n; i += 256) {
+        const uint32_t key = keys[i];
+        entries[owner * n + i] = key;
+        float c = 0.0f;
+        if (key != 0xFFFFFFFFu) c = a[(owner * kSweepTokens + ((key >> 8) & 3u)) * top_k + (key & 255u)];
+        coef[owner * n + i] = c;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSweepThreads) void expert_states_sweep_kernel(
+    const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ entries, const float* __restrict__ coef,
+    T* __restrict__ out, int64_t num_tokens, int64_t num_experts, int top_k, uint32_t row_bytes, int num_bands,
+    int token_blocks) {
+    constexpr int CL = 8, U = kBucketBatch;
+    static_assert(sizeof(T) == 2, "eight 16-bit columns per lane: a 128-byte band is 64 columns");
+    __shared__ __attribute__((aligned(16))) float sums[kSweepWgTokens * 64];   // [512 tokens][64 columns]: 128 KiB
+    const int b = (int)blockIdx.x;
+    const int band = (b & 7) + 8 * ((b >> 3) / token_blocks);           // XCD (b & 7) takes bands x, x + 8, ...
+    const int tb = (b >> 3) % token_blocks;
+    if (band >= num_bands) return;
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int c = lane & (CL - 1), group = tid / CL;                    // lane group 0..127 of the workgroup
+    const int group_base = (lane & ~(CL - 1)) << 2;
+    const int64_t owner = (int64_t)tb * (kSweepThreads / CL) + group;
+    const int n = kSweepTokens * top_k;
+    const uint32_t col_bytes = (uint32_t)band * (CL * 16) + (uint32_t)c * 16;
+    const __amdgpu_buffer_rsrc_t wr = table_resource(up, table_bytes);
+    const uint64_t list_bytes = (uint64_t)((num_tokens + kSweepTokens - 1) / kSweepTokens) * (uint64_t)n * 4u;
+    const __amdgpu_buffer_rsrc_t er = table_resource(entries, (uint32_t)list_bytes), cr = table_resource(coef, (uint32_t)list_bytes);
+    // the group's rows of `sums`: token tl at (group * 4 + tl) * 64 floats; this lane's 8 columns are two 16-byte halves,
+    // which odd groups keep in the opposite order so that two groups served together never meet in a bank
+    float* my_rows = sums + group * kSweepTokens * 64 + c * 8;
+    const int h0 = (group & 1) * 4, h1 = 4 - h0;
+    const f32x4_t zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int tl = 0; tl < kSweepTokens; ++tl) {
+        *reinterpret_cast<f32x4_t*>(my_rows + tl * 64) = zero4;
+        *reinterpret_cast<f32x4_t*>(my_rows + tl * 64 + 4) = zero4;
+    }
+    const uint32_t list_at = (uint32_t)((uint64_t)owner * (uint64_t)n * 4u);
+    auto load_entries = [&](int pos, u32x4_t (&en)[2], u32x4_t (&cf)[2]) {
+        const uint32_t at = list_at + ((uint32_t)pos + (uint32_t)c * 8u) * 4u;
+        const bool ok = pos + c * 8 < n;                                // whole 8-entry pieces: n is a multiple of 4, see below
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            en[h] = load_row_piece_streaming(er, ok ? at + 16u * h : kBadOffset);
+            cf[h] = load_row_piece_streaming(cr, ok ? at + 16u * h : kBadOffset);
+        }
+    };
+    // Four entries at a time, the gathers of the next four issued before the current four are added: the loads of a
+    // wave never drain.  `fetch` turns four entries into their keys, coefficients and row pieces; `add` adds them.
+    constexpr int Q = 4;
+    struct Quad {
+        u32x4_t w[Q];
+        uint32_t key[Q];
+        float cv[Q];
+    };
+    auto fetch = [&](Quad& q, const u32x4_t& e4, const u32x4_t& c4, int src, int at) {
+#pragma unroll
+        for (int u = 0; u < Q; ++u) {
+            const bool live = at + u < n;                           // the last piece of a list may reach into the next one
+            q.key[u] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)e4[u]);
+            const float cvu = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, (int)c4[u]));
+            q.cv[u] = live ? cvu : 0.0f;
+            const uint32_t e = q.key[u] >> 10;
+            // a key that names no expert (an id outside the table sorts to the end with coefficient 0) takes an
+            // address outside the table, which reads as zeros: 0 * row must not meet a non-finite row
+            q.w[u] = load_row_piece(wr, (e < (uint32_t)num_experts && live) ? e * row_bytes + col_bytes : kBadOffset);
+        }
+    };
+    auto add = [&](const Quad& q) {
+#pragma unroll
+        for (int u = 0; u < Q; ++u) {
+            float* row = my_rows + ((q.key[u] >> 8) & 3u) * 64;
+            f32x4_t s0 = *reinterpret_cast<f32x4_t*>(row + h0), s1 = *reinterpret_cast<f32x4_t*>(row + h1);
+            float acc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+            axpy16_coef<T>(q.cv[u], q.w[u], acc);
+            s0 = f32x4_t{acc[0], acc[1], acc[2], acc[3]};
+            s1 = f32x4_t{acc[4], acc[5], acc[6], acc[7]};
+            *reinterpret_cast<f32x4_t*>(row + h0) = s0;
+            *reinterpret_cast<f32x4_t*>(row + h1) = s1;
+        }
+    };
+    u32x4_t en[2], cf[2];
+    load_entries(0, en, cf);
+    Quad qa, qb;
+    fetch(qa, en[0], cf[0], group_base, 0);
+    for (int pos = 0; pos < n; pos += kBucketChunk) {
+        u32x4_t nen[2], ncf[2];
+        load_entries(pos + kBucketChunk, nen, ncf);                     // the next 64 entries, ahead of time
+#pragma unroll 1
+        for (int bt = 0; bt < kBucketChunk / 8; ++bt) {
+            const int at = pos + bt * 8;
+            if (at >= n) break;
+            const int src = group_base + bt * 4;                        // lane bt of the group holds entries at .. at + 7
+            fetch(qb, en[1], cf[1], src, at + 4);
+            add(qa);
+            // the first four of the next eight: from lane bt + 1, or from lane 0 of the next 64
+            if (bt + 1 < kBucketChunk / 8) fetch(qa, en[0], cf[0], src + 4, at + 8);
+            else fetch(qa, nen[0], ncf[0], group_base, at + 8);
+            add(qb);
+            // every list has the same length, so equal positions mean (statistically) equal experts: keeping the
+            // workgroup's waves within two batches of each other keeps their gathers inside one window of the band
+            if (bt & 1) __syncthreads();
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            en[h] = nen[h];
+            cf[h] = ncf[h];
+        }
+    }
+    // the group's tokens: 8 columns per lane, rounded once
+#pragma unroll
+    for (int tl = 0; tl < kSweepTokens; ++tl) {
+        const int64_t t = owner * kSweepTokens + tl;
+        if (t < num_tokens) {
+            const f32x4_t s0 = *reinterpret_cast<f32x4_t*>(my_rows + tl * 64 + h0), s1 = *reinterpret_cast<f32x4_t*>(my_rows + tl * 64 + h1);
+            const float acc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+            *reinterpret_cast<u32x4_t*>(reinterpret_cast<char*>(out) + t * (int64_t)row_bytes + col_bytes) = pack16<T>(acc);
+        }
+    }
+}
+
 struct BucketedPlan {
     int chunk_lanes, num_bands, parts, blocks_per_unit;
     unsigned grid;
-    size_t off_bucket, off_offsets, off_pairs, off_tok, off_exp, off_a, off_spart, off_xb, bytes;
+    size_t off_bucket, off_offsets, off_pairs, off_tok, off_exp, off_a, off_spart, off_xb, off_sweep_keys, off_sweep_coef, bytes;
+    bool sweep;
 };
+
+// The sweep needs 16-bit rows of whole 128-byte bands, at most 256 pairs per token, ids below 2^22 and lists below 4 GiB.
+bool sweep_possible(int64_t T_, int H, int64_t E, int K, size_t elt) {
+    const int64_t padded = (T_ + kSweepTokens - 1) / kSweepTokens * kSweepTokens;
+    return elt == 2 && (H * elt) % 128 == 0 && K <= kSweepMaxTopK && E <= (1ll << 22) && padded * K * 4 < (int64_t)kBadOffset;
+}
 
 // Band width: as wide as lets the band of all tokens stay in one XCD's L2 (about 2 MiB of its 4), at least 128 bytes.
 BucketedPlan plan_bucketed(int64_t T_, int H, int64_t E, int K, size_t elt) {
@@ -733,6 +928,10 @@ BucketedPlan plan_bucketed(int64_t T_, int H, int64_t E, int K, size_t elt) {
     p.off_a = take((size_t)pairs * 4);
     p.off_spart = take((size_t)p.num_bands * pairs * 4);
     p.off_xb = take((size_t)T_ * H * elt);
+    p.sweep = sweep_possible(T_, H, E, K, elt);
+    const size_t padded_pairs = (size_t)((T_ + kSweepTokens - 1) / kSweepTokens * kSweepTokens) * (size_t)K;
+    p.off_sweep_keys = take(p.sweep ? padded_pairs * 4 : 0);
+    p.off_sweep_coef = take(p.sweep ? padded_pairs * 4 : 0);
     p.bytes = o;
     return p;
 }
@@ -790,6 +989,24 @@ int launch_expert_bucketed(int act, const void* x, const void* down, const void*
         hipLaunchKernelGGL((expert_gate_sorted_kernel<T, kActGelu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
                            pairs, (const T*)gates, (const int32_t*)sorted_pairs, (const int32_t*)offsets, E, a, p.num_bands);
     FMOE_CHECK_LAUNCH("fmoe_expert_forward(bucketed gate)");
+    if constexpr (sizeof(T) == 2) {
+        if (p.sweep) {
+            uint32_t* keys = (uint32_t*)(ws + p.off_sweep_keys);
+            float* coef = (float*)(ws + p.off_sweep_coef);
+            const int64_t owners = (T_ + kSweepTokens - 1) / kSweepTokens;
+            hipLaunchKernelGGL(expert_owner_sort_kernel, dim3((unsigned)owners), dim3(256), 0, stream, indices, (const float*)a,
+                               keys, coef, T_, E, K);
+            FMOE_CHECK_LAUNCH("fmoe_expert_forward(owner sort)");
+            const int bands = (int)(row_bytes / 128);
+            const int token_blocks = (int)((T_ + kSweepWgTokens - 1) / kSweepWgTokens);
+            const unsigned grid = (unsigned)(8 * token_blocks * ((bands + 7) / 8));
+            hipLaunchKernelGGL((expert_states_sweep_kernel<T>), dim3(grid), dim3(kSweepThreads), 0, stream, (const T*)up,
+                               table_bytes, (const uint32_t*)keys, (const float*)coef, (T*)out, T_, E, K, row_bytes, bands,
+                               token_blocks);
+            FMOE_CHECK_LAUNCH("fmoe_expert_forward(sweep)");
+            return FMOE_OK;
+        }
+    }
     return launch_expert_rows_coef<T>(up, indices, a, T_, H, E, K, out, stream);
 }
 
