@@ -47,7 +47,7 @@ int router_forward_impl(const void* x, const void* gate_w, void* running_mean, v
                         int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
                         void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
                         uint32_t* row_offsets, uint32_t row_bytes, void* workspace, size_t workspace_bytes,
-                        hipStream_t stream);
+                        hipStream_t stream, int split_query = 0);
 
 // Column-slice schedule of the routed experts on row offsets that are already in place at the start of `workspace`
 // (the layout fmoe_expert_workspace_bytes describes); defined in fmoe_expert.hip.

@@ -781,7 +781,7 @@ __global__ __launch_bounds__(kSweepThreads) void expert_states_sweep_kernel(
     const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ entries, const float* __restrict__ coef,
     T* __restrict__ out, int64_t num_tokens, int64_t num_experts, int top_k, uint32_t row_bytes, int num_bands,
     int token_blocks) {
-    constexpr int CL = 8, U = kBucketBatch;
+    constexpr int CL = 8;
     static_assert(sizeof(T) == 2, "eight 16-bit columns per lane: a 128-byte band is 64 columns");
     __shared__ __attribute__((aligned(16))) float sums[kSweepWgTokens * 64];   // [512 tokens][64 columns]: 128 KiB
     const int b = (int)blockIdx.x;

@@ -246,11 +246,13 @@ template <> __device__ inline u32x4_t normalise16<f16_t>(u32x4_t raw, const floa
 constexpr int kGatePrefetch = 3;
 constexpr int kGateMaxK = 8192;     // mean / rstd of all k are staged in LDS once: 2 * 4 * K bytes
 
+// split != 0: half h of the outputs (columns [h*N/2, (h+1)*N/2)) scores only half h of the normalised activations,
+// w is [N, K/2]: the product-key form in which each sub-key table sees its own half of the query (a block-diagonal gate).
 template <typename T>
 __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const float* __restrict__ mean_rstd, float* __restrict__ logits32,
-                                                          T* __restrict__ logits, int M, int N, int K, int tiles_m,
-                                                          int tiles_n) {
+                                                          T* __restrict__ logits, int M, int N, int K_full, int tiles_m,
+                                                          int tiles_n, int split) {
     using Frag = typename Mfma32<T>::Frag;
     constexpr int BM = 64, BN = 64, CH = 2;   // CH = 16-byte packets per thread per tile and operand
     constexpr int D = kGatePrefetch;
@@ -265,11 +267,14 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ 
     const int ch = tid % kTileChunks;          // this thread's packet column inside a k-tile: the same for all its packets
     const int row0 = tid / kTileChunks;        // rows row0 and row0 + 32
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    // the k range of this tile: all of it, or the half of the activations its columns score (tiles do not straddle halves)
+    const int K = split ? K_full / 2 : K_full;
+    const int k_off = (split && n0 >= N / 2) ? K : 0;
     const int k_tiles = (K + kTileK - 1) / kTileK;
     const int kpad = k_tiles * kTileK;
     for (int i = tid; i < kpad; i += 256) {
-        stats[i] = i < K ? mean_rstd[i] : 0.0f;
-        stats[kpad + i] = i < K ? mean_rstd[K + i] : 0.0f;
+        stats[i] = i < K ? mean_rstd[k_off + i] : 0.0f;
+        stats[kpad + i] = i < K ? mean_rstd[K_full + k_off + i] : 0.0f;
     }
     u32x4_t ra[D][CH], rb[D][CH];
 
@@ -279,7 +284,7 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ 
 #pragma unroll
         for (int it = 0; it < CH; ++it) {
             const int gm = m0 + row0 + it * 32, gn = n0 + row0 + it * 32;
-            ra[slot][it] = (gm < M && k_ok) ? *reinterpret_cast<const u32x4_t*>(x + (int64_t)gm * K + gk) : zero4;
+            ra[slot][it] = (gm < M && k_ok) ? *reinterpret_cast<const u32x4_t*>(x + (int64_t)gm * K_full + k_off + gk) : zero4;
             rb[slot][it] = (gn < N && k_ok) ? *reinterpret_cast<const u32x4_t*>(w + (int64_t)gn * K + gk) : zero4;
         }
     };
@@ -340,19 +345,21 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ 
 __global__ __launch_bounds__(256) void router_gate_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                               const float* __restrict__ mean_rstd,
                                                               float* __restrict__ logits32, float* __restrict__ logits,
-                                                              int M, int N, int K) {
+                                                              int M, int N, int K_full, int split) {
     constexpr int TS = 64, KS = 16;
     __shared__ float As[KS][TS + 1];
     __shared__ float Bs[KS][TS + 1];
     const int m0 = blockIdx.y * TS, n0 = blockIdx.x * TS;
     const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    const float* mean = mean_rstd;
-    const float* rstd = mean_rstd + K;
+    const int K = split ? K_full / 2 : K_full;              // split: the tile's columns score one half of the activations
+    const int k_off = (split && n0 >= N / 2) ? K : 0;
+    const float* mean = mean_rstd + k_off;
+    const float* rstd = mean_rstd + K_full + k_off;
     float acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += KS) {
         for (int q = threadIdx.x; q < TS * KS; q += 256) {
             const int r = q / KS, kk = q % KS, gk = k0 + kk;
-            As[kk][r] = (m0 + r < M && gk < K) ? (x[(int64_t)(m0 + r) * K + gk] - mean[gk]) * rstd[gk] : 0.0f;
+            As[kk][r] = (m0 + r < M && gk < K) ? (x[(int64_t)(m0 + r) * K_full + k_off + gk] - mean[gk]) * rstd[gk] : 0.0f;
             Bs[kk][r] = (n0 + r < N && gk < K) ? w[(int64_t)(n0 + r) * K + gk] : 0.0f;
         }
         __syncthreads();
@@ -719,6 +726,18 @@ extern "C" int fmoe_router_forward(const void* x, const void* gate_w, void* runn
                                      workspace_bytes, (hipStream_t)stream);
 }
 
+extern "C" int fmoe_router_forward_split(const void* x, const void* sub_keys, void* running_mean, void* running_var,
+                                         int64_t* num_batches_tracked, int stats_dtype, int training, float momentum,
+                                         float eps, int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype,
+                                         int norm_topk_prob, void* router_logits, float* logits_fp32, float* scores,
+                                         int64_t* indices, void* gates, void* workspace, size_t workspace_bytes, void* stream) {
+    fmoe::clear_error();
+    return fmoe::router_forward_impl(x, sub_keys, running_mean, running_var, num_batches_tracked, stats_dtype, training,
+                                     momentum, eps, num_tokens, hidden, num_keys, top_k, dtype, norm_topk_prob,
+                                     router_logits, logits_fp32, scores, indices, gates, nullptr, 0u, workspace,
+                                     workspace_bytes, (hipStream_t)stream, 1);
+}
+
 extern "C" int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running_mean, void* running_var,
                                            int64_t* num_batches_tracked, int stats_dtype, int training, float momentum,
                                            float eps, int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype,
@@ -745,8 +764,10 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
                               int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
                               void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
                               uint32_t* row_offsets, uint32_t row_bytes, void* workspace, size_t workspace_bytes,
-                              hipStream_t s) {
+                              hipStream_t s, int split_query) {
     using namespace fmoe;
+    FMOE_REQUIRE(!split_query || (num_keys % 64 == 0 && hidden % 2 == 0), FMOE_ERR_UNSUPPORTED,
+                 "fmoe_router_forward_split: num_keys=%d must be a multiple of 64 and hidden=%d even", num_keys, hidden);
     FMOE_REQUIRE(dtype_ok(dtype) && dtype_ok(stats_dtype), FMOE_ERR_BAD_DTYPE,
                  "fmoe_router_forward: unknown dtype %d / statistics dtype %d", dtype, stats_dtype);
     FMOE_REQUIRE(num_tokens >= 0 && hidden > 0 && num_keys > 0, FMOE_ERR_BAD_SHAPE,
@@ -767,8 +788,9 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
     FMOE_REQUIRE(training || (running_mean && running_var), FMOE_ERR_NULL_POINTER,
                  "fmoe_router_forward: evaluation mode needs running statistics");
     const int vec = (int)(16 / dtype_size(dtype));
-    FMOE_REQUIRE(hidden % vec == 0 && aligned16(x) && aligned16(gate_w), FMOE_ERR_ALIGNMENT,
-                 "fmoe_router_forward: hidden=%d must be a multiple of %d and tensors 16-byte aligned", hidden, vec);
+    FMOE_REQUIRE(hidden % (split_query ? 2 * vec : vec) == 0 && aligned16(x) && aligned16(gate_w), FMOE_ERR_ALIGNMENT,
+                 "fmoe_router_forward: hidden=%d must be a multiple of %d and tensors 16-byte aligned", hidden,
+                 split_query ? 2 * vec : vec);
     const ProloguePlan p = plan_prologue(num_tokens, hidden, num_keys);
     FMOE_REQUIRE(workspace_bytes >= p.bytes && aligned16(workspace), FMOE_ERR_WORKSPACE,
                  "fmoe_router_forward: workspace of %zu bytes needed, %zu given", p.bytes, workspace_bytes);
@@ -795,18 +817,18 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
     const int M = (int)num_tokens, N = 2 * num_keys;
     if (dtype == FMOE_F32) {
         hipLaunchKernelGGL(router_gate_f32_kernel, dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, s, (const float*)x,
-                           (const float*)gate_w, (const float*)mean_rstd, logits32, (float*)router_logits, M, N, hidden);
+                           (const float*)gate_w, (const float*)mean_rstd, logits32, (float*)router_logits, M, N, hidden, split_query);
     } else {
         const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
         const size_t stats_bytes = (size_t)((hidden + kTileK - 1) / kTileK) * kTileK * 2 * sizeof(float);
         if (dtype == FMOE_BF16)
             hipLaunchKernelGGL((router_gate_kernel<bf16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
                                (const bf16_t*)x, (const bf16_t*)gate_w, (const float*)mean_rstd, logits32,
-                               (bf16_t*)router_logits, M, N, hidden, tiles_m, tiles_n);
+                               (bf16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query);
         else
             hipLaunchKernelGGL((router_gate_kernel<f16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
                                (const f16_t*)x, (const f16_t*)gate_w, (const float*)mean_rstd, logits32,
-                               (f16_t*)router_logits, M, N, hidden, tiles_m, tiles_n);
+                               (f16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query);
     }
     FMOE_CHECK_LAUNCH("fmoe_router_forward(gate)");
     if (top_k == 0) return FMOE_OK;

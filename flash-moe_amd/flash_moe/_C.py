@@ -33,6 +33,8 @@ SIGNATURES = {
     "fmoe_router_workspace_bytes": (_sz, [_i64, _int, _int]),
     "fmoe_router_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int,
                                    _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "fmoe_router_forward_split": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int,
+                                         _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "fmoe_router_forward_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _int, ctypes.c_float, ctypes.c_float, _i64, _int, _int,
                                            _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
     "fmoe_expert_workspace_bytes": (_sz, [_i64, _int, _i64, _int, _int]),

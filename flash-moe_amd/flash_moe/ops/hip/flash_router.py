@@ -54,10 +54,12 @@ def router_topk_gates(
     return scores, indices, gates
 
 
-def check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok):
+def check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok, split_query=False):
     """Argument checks of the fused routing stage; returns ``(device, training)``."""
-    if tokens.dim() != 2 or gate_weight.shape != (2 * num_expert_keys, tokens.shape[1]):
-        raise ValueError("expected tokens [T, H] and a router gate weight [2*num_expert_keys, H]")
+    width = tokens.shape[1] // 2 if split_query else tokens.shape[1]
+    if tokens.dim() != 2 or gate_weight.shape != (2 * num_expert_keys, width):
+        raise ValueError("expected tokens [T, H] and a router gate weight [2*num_expert_keys, H] "
+                         "([2*num_expert_keys, H/2] sub-key tables with split_query)")
     assert 0 <= num_experts_per_tok <= num_expert_keys, (
         f"num_experts_per_tok should be in [0, {num_expert_keys}], but got {num_experts_per_tok}"
     )
@@ -76,7 +78,7 @@ def check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_pe
 
 def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.nn.BatchNorm1d, num_expert_keys: int,
                    num_experts_per_tok: int, norm_topk_prob: bool = False, return_logits32: bool = False,
-                   return_stats: bool = False):
+                   return_stats: bool = False, split_query: bool = False):
     """The block's whole routing stage in one call of ``fmoe_router_forward``: batch-norm (training or evaluation
     mode, taken from ``norm.training``; its running statistics are updated in place), the router gate, the per-half
     log-softmax, the product-key top-k and the gates (flash_moe/modules/flash_moe.py:62-85).
@@ -84,8 +86,10 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
     Returns ``(router_logits [T, 2*nk] in tokens.dtype, scores [T,K] fp32, indices [T,K] int64, gates [T,K] in
     tokens.dtype)``, plus the fp32 logits the routing was computed from when ``return_logits32`` is set, plus the
     batch-norm mean and 1/sqrt(var + eps) used ([2*H] fp32, a view of the call's workspace) when ``return_stats`` is set.
+    ``split_query``: ``gate_weight`` is two sub-key tables [2*nk, H/2], each scoring its own half of the normalised query
+    (``fmoe_router_forward_split``; equal to a block-diagonal [2*nk, H] gate); the module never uses this form.
     """
-    dev, training = check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok)
+    dev, training = check_router_args(tokens, gate_weight, norm, num_expert_keys, num_experts_per_tok, split_query)
     T, H = tokens.shape
     x, w = tokens.contiguous(), gate_weight.contiguous()
     K = num_experts_per_tok
@@ -99,7 +103,7 @@ def router_forward(tokens: torch.Tensor, gate_weight: torch.Tensor, norm: torch.
     ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
     rm, rv, nbt = norm.running_mean, norm.running_var, norm.num_batches_tracked
     with torch.cuda.device(dev):
-        status = L.fmoe_router_forward(
+        status = (L.fmoe_router_forward_split if split_query else L.fmoe_router_forward)(
             _C.ptr(x), _C.ptr(w), _C.ptr(rm), _C.ptr(rv), _C.ptr(nbt), _C.dtype_code(rm.dtype), int(training),
             float(norm.momentum), float(norm.eps), T, H, num_expert_keys, K, _C.dtype_code(x.dtype),
             int(bool(norm_topk_prob)), _C.ptr(logits), _C.ptr(logits32), _C.ptr(scores), _C.ptr(indices), _C.ptr(gates),

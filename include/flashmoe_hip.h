@@ -95,6 +95,20 @@ int fmoe_router_forward(const void* x, const void* gate_w, void* running_mean, v
                         void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same routing stage with a split query: half h of the gate (sub_keys rows [h*nk, (h+1)*nk), each of hidden/2
+ * columns) scores only columns [h*hidden/2, (h+1)*hidden/2) of the normalised activations, i.e. fmoe_router_forward with a
+ * block-diagonal router_gate.weight, at half the multiply-adds.  This is the product-key form in which each sub-key
+ * table sees its own half of the query (two 128 x 512 tables against a 1024-wide query in the router benchmark
+ * configuration); FlashMoE.forward itself scores the full query against both halves (flash_moe/modules/flash_moe.py:65-66),
+ * so the module never takes this entry point.
+ *   sub_keys [2*nk, H/2] dtype; everything else as in fmoe_router_forward.  Requires nk % 64 == 0 and H/2 a whole number
+ *   of 16-byte packets. */
+int fmoe_router_forward_split(const void* x, const void* sub_keys, void* running_mean, void* running_var,
+                              int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
+                              int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
+                              void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
 /* fmoe_router_forward for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same results.  It has no
  * counterpart in the reference.  The scratch the call needs (batch-norm partials, mean and 1/std: about 6 MiB) is a

@@ -100,7 +100,12 @@ def test_expert_argument_checks():
     assert sliced >= 4096 * 64 * (4 + 4 + 8 * 4) and sliced % 256 == 0               # 8 slices of 256 bytes
     wide = lib.fmoe_expert_workspace_bytes(4096, 1024, 32768, 64, _C.BF16)
     assert wide >= 4096 * 64 * (4 + 4 + 16 * 4) and wide % 256 == 0                   # 16 slices of 128 bytes
-    assert lib.fmoe_expert_workspace_bytes(32768, 2048, 262144, 128, _C.BF16) == 0      # table slice too large for L2
+    # a table whose slices are too large for L2 takes the bucketed schedule: bucketing state, grouped order, band-major x,
+    # 32 bands of partial scores, the per-owner lists of the sweep
+    big = lib.fmoe_expert_workspace_bytes(32768, 2048, 262144, 128, _C.BF16)
+    assert big >= 32768 * 128 * 4 * (4 + 32 + 2) + 32768 * 2048 * 2 and big % 256 == 0
+    assert big == lib.fmoe_expert_workspace_bytes_algo(32768, 2048, 262144, 128, _C.BF16, _C.EXPERT_BUCKETS)
+    assert lib.fmoe_expert_workspace_bytes_algo(32768, 2048, 262144, 128, _C.BF16, _C.EXPERT_ROWS) == 0
     assert lib.fmoe_expert_workspace_bytes(64, 1024, 16384, 8, _C.BF16) == 0            # too few pairs
     assert lib.fmoe_expert_workspace_bytes_algo(64, 1024, 16384, 8, _C.BF16, _C.EXPERT_SLICES) > 0
     assert lib.fmoe_expert_workspace_bytes_algo(4096, 1024, 16384, 64, _C.BF16, _C.EXPERT_ROWS) == 0

@@ -226,3 +226,40 @@ def test_fused_router_rejects_single_token_in_training():
     bn.eval()
     out = router_forward(torch.randn(1, 64, device="cuda"), torch.randn(16, 64, device="cuda"), bn, 8, 4)
     assert out[2].shape == (1, 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,nk,K", [(8192, 1024, 128, 64), (300, 256, 64, 16)])
+def test_split_query_router_equals_a_block_diagonal_gate(dtype, T, H, nk, K):
+    """Two sub-key tables [nk, H/2], each scoring its own half of the query (the router benchmark configuration as worded),
+    against the general routing stage with the block-diagonal gate they stand for: the zero blocks add exact zeros, so
+    logits, scores and indices agree bit for bit; and the logits against the oracle's prologue on that gate."""
+    from flash_moe.ops.hip.flash_router import router_forward
+
+    g = torch.Generator().manual_seed(T + H)
+    x = (torch.randn(T, H, generator=g) * 1.2 + 0.1).to(dtype)
+    tables = (torch.randn(2 * nk, H // 2, generator=g) * 0.02).to(dtype)
+    dense = torch.zeros(2 * nk, H, dtype=dtype)
+    dense[:nk, : H // 2] = tables[:nk]
+    dense[nk:, H // 2:] = tables[nk:]
+
+    def run(weight, split):
+        bn = torch.nn.BatchNorm1d(H, affine=False).to(device="cuda", dtype=dtype)
+        return router_forward(x.cuda(), weight.cuda(), bn, nk, K, True, return_logits32=True, split_query=split), bn
+
+    (logits, scores, indices, gates, logits32), bn = run(tables, True)
+    (d_logits, d_scores, d_indices, d_gates, d_logits32), d_bn = run(dense, False)
+    assert torch.equal(logits32, d_logits32) and torch.equal(logits, d_logits)
+    assert torch.equal(scores, d_scores) and torch.equal(indices, d_indices) and torch.equal(gates, d_gates)
+    assert torch.equal(bn.running_mean, d_bn.running_mean) and torch.equal(bn.running_var, d_bn.running_var)
+    ref_logits, _ = orc.router_prologue(x.float(), dense.float(), nk)
+    tol = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 2e-2}[dtype]
+    torch.testing.assert_close(logits.float().cpu().view(T, 2, nk).transpose(0, 1), ref_logits, rtol=tol, atol=tol)
+    # each half only sees its half of the query: changing the other half of x leaves its logits untouched (eval mode,
+    # so that the statistics of the untouched columns stay what they were)
+    x2 = x.clone()
+    x2[:, H // 2:] += 1.0
+    bn_e = torch.nn.BatchNorm1d(H, affine=False).to(device="cuda", dtype=dtype).eval()
+    a = router_forward(x.cuda(), tables.cuda(), bn_e, nk, K, False, return_logits32=True, split_query=True)[4]
+    b = router_forward(x2.cuda(), tables.cuda(), bn_e, nk, K, False, return_logits32=True, split_query=True)[4]
+    assert torch.equal(a[:, :nk], b[:, :nk]) and not torch.equal(a[:, nk:], b[:, nk:])
