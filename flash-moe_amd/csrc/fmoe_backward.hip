@@ -12,9 +12,9 @@
 // No floating-point atomics on global memory: every output element is written once and sums run in a fixed order
 // (pairs of an expert in ascending pair index), so gradients are reproducible bit for bit.  The per-token part of the
 // expert backward is one wave per token with the token's rows of x and dout in registers (the layout of the forward
-// row kernel).  The per-expert part needs the pairs grouped by expert: a counting sort (integer histogram, exclusive
-// scan, fill through per-expert cursors) puts each expert's pairs in one segment in arbitrary order, and the wave that
-// owns the expert walks its segment in ascending pair index by repeatedly taking the smallest index not yet used.
+// row kernel).  The per-expert part needs the pairs grouped by expert: the bucketing stage (fmoe_bucket.hip: integer
+// histogram taken by the per-token kernels, scan, fill, ordering pass) gives each expert one segment listing its pairs in
+// ascending pair index, and the wave that owns the expert walks it in that order.
 #include "fmoe_common.h"
 #include "fmoe_vec.h"
 
@@ -319,61 +319,6 @@ __global__ __launch_bounds__(256) void expert_backward_gate_kernel(
     if (valid) atomicAdd(&counts[indices[p]], 1);   // integer histogram: the result does not depend on order
 }
 
-__global__ void zero_i32_kernel(int32_t* __restrict__ p, int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = 0;
-}
-
-// offsets[e] = number of pairs of experts < e, for e in [0, num_experts]; one workgroup.  The counts are taken in tiles
-// of kScanThreads * 4 (coalesced 16-byte loads, four counts per thread), each tile scanned across the workgroup with the
-// running total carried from tile to tile.
-constexpr int kScanThreads = 1024;
-__global__ __launch_bounds__(kScanThreads) void expert_scan_kernel(const int32_t* __restrict__ counts,
-                                                                  int32_t* __restrict__ offsets, int64_t num_experts) {
-    __shared__ int32_t wave_total[kScanThreads / kWave];
-    __shared__ int32_t carry_s;
-    const int tid = (int)threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-    if (tid == 0) carry_s = 0;
-    __syncthreads();
-    for (int64_t base = 0; base < num_experts; base += kScanThreads * 4) {
-        const int64_t e0 = base + (int64_t)tid * 4;
-        int32_t c[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) c[j] = e0 + j < num_experts ? counts[e0 + j] : 0;
-        const int32_t mine = c[0] + c[1] + c[2] + c[3];
-        int32_t incl = mine;
-#pragma unroll
-        for (int d = 1; d < kWave; d <<= 1) {
-            const int32_t up = __shfl_up(incl, d, kWave);
-            if (lane >= d) incl += up;
-        }
-        if (lane == kWave - 1) wave_total[wave] = incl;
-        __syncthreads();
-        int32_t before = carry_s;
-        for (int w = 0; w < wave; ++w) before += wave_total[w];
-        int32_t run = before + incl - mine;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (e0 + j < num_experts) offsets[e0 + j] = run;
-            run += c[j];
-        }
-        __syncthreads();
-        if (tid == kScanThreads - 1) carry_s = run;      // the last thread's running total is the tile's inclusive total
-        __syncthreads();
-    }
-    if (tid == 0) offsets[num_experts] = carry_s;
-}
-
-// pairs[offsets[e] + (arrival order)] = p for every valid pair: segments are complete, their internal order is not fixed
-__global__ __launch_bounds__(256) void expert_fill_kernel(const int64_t* __restrict__ indices, const int32_t* __restrict__ offsets,
-                                                          int32_t* __restrict__ cursor, uint32_t* __restrict__ pairs,
-                                                          int64_t num_pairs, int64_t num_experts) {
-    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (p >= num_pairs) return;
-    const int64_t e = indices[p];
-    if (e < 0 || e >= num_experts) return;
-    pairs[offsets[e] + atomicAdd(&cursor[e], 1)] = (uint32_t)p;
-}
-
 // One wave per expert: its rows of ddown and dup, summed over its pairs in ascending pair index.
 template <typename T, int NCH>
 __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kernel(
@@ -398,39 +343,10 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
 
     const int begin = offsets[e], end = offsets[e + 1];
     const int n_total = end - begin;
-    // The segment is walked in ascending pair index, kWave pairs per round: the round takes the kWave smallest indices
-    // above the last one used.  Segments of at most kWave pairs (the usual case) are read once.
-    uint32_t floor_excl = 0;     // pairs with index < floor_excl are done (pair indices are distinct)
+    // The segment lists the expert's pairs in ascending pair index (the bucketing stage orders it), kWave pairs per round.
     for (int done = 0; done < n_total; done += kWave) {
         const int n = n_total - done < kWave ? n_total - done : kWave;
-        uint32_t mine = 0xFFFFFFFFu;   // this lane's pair of the round: the (lane)-th smallest index >= floor_excl
-        if (n_total <= kWave) {
-            // rank of each pair inside the segment by counting smaller ones
-            const uint32_t p = lane < n_total ? pairs[begin + lane] : 0xFFFFFFFFu;
-            int rank = 0;
-            for (int j = 0; j < n_total; ++j) rank += ((uint32_t)__builtin_amdgcn_readlane((int)p, j) < p) ? 1 : 0;
-            // lane `rank` takes p: a permutation of the live lanes
-            const int got = __builtin_amdgcn_ds_permute(rank << 2, (int)p);
-            mine = lane < n_total ? (uint32_t)got : 0xFFFFFFFFu;
-        } else {
-            // long segment: kWave selection passes over it, each taking the smallest remaining index
-            uint32_t last = floor_excl;
-            for (int r = 0; r < n; ++r) {
-                uint32_t best = 0xFFFFFFFFu;
-                for (int j = lane; j < n_total; j += kWave) {
-                    const uint32_t p = pairs[begin + j];
-                    if (p >= last && p < best) best = p;
-                }
-#pragma unroll
-                for (int d = 32; d >= 1; d >>= 1) {
-                    const uint32_t o = (uint32_t)__shfl_xor((int)best, d, kWave);
-                    best = o < best ? o : best;
-                }
-                if (lane == r) mine = best;
-                last = best + 1;
-            }
-            floor_excl = last;
-        }
+        const uint32_t mine = lane < n ? pairs[begin + done + lane] : 0u;
         uint32_t tok = 0;
         float cu = 0.0f, cd = 0.0f;
         if (lane < n) {
@@ -488,8 +404,8 @@ ExpertBwdPlan plan_expert_backward(int64_t T_, int H, int64_t E, int K, int dtyp
     p.off_coef_up = take(pairs * 4);
     p.off_coef_down = take(pairs * 4);
     p.off_pairs = take(pairs * 4);
-    p.off_counts = take((size_t)E * 4);        // counts and cursor are adjacent: one clearing launch
-    p.off_cursor = take((size_t)E * 4);
+    p.off_counts = take(bucket_workspace_bytes(E));     // per-expert counts, then the fill's cursors, and the scan state
+    p.off_cursor = p.off_counts;
     p.off_offsets = take((size_t)(E + 1) * 4);
     p.slices = expert_slices_usable(T_, H, E, K, dtype);
     p.num_slices = p.slices ? expert_slice_count(T_, H, E, K, dtype) : 0;
@@ -513,8 +429,8 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
     float* coef_up = (float*)(ws + p.off_coef_up);
     float* coef_down = (float*)(ws + p.off_coef_down);
     uint32_t* pairs_by_expert = (uint32_t*)(ws + p.off_pairs);
-    int32_t* counts = (int32_t*)(ws + p.off_counts);
-    int32_t* cursor = (int32_t*)(ws + p.off_cursor);
+    void* bucket_ws = ws + p.off_counts;
+    int32_t* counts = bucket_counts(bucket_ws);
     int32_t* offsets = (int32_t*)(ws + p.off_offsets);
     const int64_t pairs = T_ * K;
     const int nch = (H / V + kWave - 1) / kWave;
@@ -522,9 +438,7 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
     const dim3 token_grid((unsigned)((T_ + kBwdWaves - 1) / kBwdWaves));
     const dim3 expert_grid((unsigned)((E + kBwdWaves - 1) / kBwdWaves));
 
-    const int64_t clear = (int64_t)((p.off_cursor - p.off_counts) / 4) + E;
-    hipLaunchKernelGGL(zero_i32_kernel, dim3(256), dim3(256), 0, stream, counts, clear);
-    FMOE_CHECK_LAUNCH("fmoe_expert_backward(clear)");
+    if (int rc = bucket_clear(bucket_ws, E, stream)) return rc;
     if (p.slices) {
         uint32_t* off32 = (uint32_t*)(ws + p.off_off32);
         float* spart_s = (float*)(ws + p.off_spart_s);
@@ -550,11 +464,10 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
         FMOE_CHECK_LAUNCH("fmoe_expert_backward(tokens)");
     }
 
-    hipLaunchKernelGGL(expert_scan_kernel, dim3(1), dim3(kScanThreads), 0, stream, (const int32_t*)counts, offsets, E);
-    FMOE_CHECK_LAUNCH("fmoe_expert_backward(scan)");
-    hipLaunchKernelGGL(expert_fill_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, indices,
-                       (const int32_t*)offsets, cursor, pairs_by_expert, pairs, E);
-    FMOE_CHECK_LAUNCH("fmoe_expert_backward(fill)");
+    // the per-token kernels above counted the pairs of every expert: offsets, segments, each in ascending pair index
+    if (int rc = bucket_scan_fill(indices, bucket_ws, pairs, E, K, offsets, (int32_t*)pairs_by_expert, nullptr, 1u, nullptr, 1u,
+                                  nullptr, 0, 1, stream))
+        return rc;
 
 #define FMOE_LAUNCH_WEIGHT(N)                                                                                            \
     hipLaunchKernelGGL((expert_backward_weight_kernel<T, N>), expert_grid, block, 0, stream, (const T*)dout, (const T*)x, \

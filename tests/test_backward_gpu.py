@@ -434,3 +434,49 @@ def test_router_prologue_backward(dtype, training, T, H, nk):
     assert rel_fro(wd.grad, w64.grad) < tol, f"dgate {rel_fro(wd.grad, w64.grad):.3e}"
     if training:   # a constant shift of the loss gradient along tokens cannot change dx: columns of dx sum to ~0
         assert float(xd.grad.float().sum(0).abs().max()) < 50 * tol * float(xd.grad.float().abs().max()) * T ** 0.5
+
+
+def test_expert_backward_with_skewed_routing_is_exact_and_quick():
+    """One expert selected by every one of 8192 tokens (a segment of 8192 pairs, as early in training or after a router
+    collapse) next to ordinary experts: gradients against float64, bit-reproducible, and the call stays in the range of
+    an ordinary backward (the long segment is walked once, in order)."""
+    import time
+
+    from flash_moe.ops.hip.flash_expert import expert_backward
+
+    T, H, E, K = 8192, 1024, 4096, 8
+    g = gen(31)
+    x = torch.randn(T, H, generator=g).bfloat16()
+    wd = (torch.randn(E, H, generator=g) * 0.05).bfloat16()
+    wu = (torch.randn(E, H, generator=g) * 0.05).bfloat16()
+    idx = torch.stack([torch.randperm(E - 1, generator=g)[:K] + 1 for _ in range(T)])
+    idx[:, 3] = 0                                                # every token also selects expert 0
+    gates = torch.softmax(torch.randn(T, K, generator=g), -1).bfloat16()
+    dout = (torch.randn(T, H, generator=g) * 0.1).bfloat16()
+    args = tuple(t.cuda() for t in (dout, x, wd, wu, idx, gates))
+    got = expert_backward(*args)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    again = expert_backward(*args)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+    assert elapsed < 0.05, f"{elapsed * 1e3:.1f} ms for a backward with one 8192-pair segment"
+    # the hot expert's rows against float64: ddown[0] = sum_t ds_t x_t, dup[0] = sum_t silu(s_t) g_t dout_t
+    x64, wd64, wu64, g64, do64 = (t.double() for t in (x, wd, wu, gates, dout))
+    s = x64 @ wd64[0]
+    sig = torch.sigmoid(s)
+    act = s * sig
+    u = do64 @ wu64[0]
+    ds = u * g64[:, 3] * (sig * (1 + s * (1 - sig)))
+    assert rel_fro(got[1][0], ds @ x64) < 1.5e-2
+    assert rel_fro(got[2][0], (act * g64[:, 3]) @ do64) < 1.5e-2
+    # an ordinary expert's rows too
+    e = int(idx[5, 0])
+    sel = (idx == e)
+    tok, slot = sel.nonzero(as_tuple=True)
+    s_e = x64[tok] @ wd64[e]
+    sig_e = torch.sigmoid(s_e)
+    u_e = do64[tok] @ wu64[e]
+    assert rel_fro(got[2][e], (s_e * sig_e * g64[tok, slot]) @ do64[tok]) < 1.5e-2
+    assert rel_fro(got[1][e], (u_e * g64[tok, slot] * (sig_e * (1 + s_e * (1 - sig_e)))) @ x64[tok]) < 1.5e-2

@@ -222,6 +222,60 @@ def test_block_c5_full_size_sampled_tokens():
     assert_output_close(y[pick], y64.to(dtype), dtype, "C5 block output vs float64 oracle on sampled tokens")
 
 
+def test_block_c5_full_size_train_mode_batch_statistics():
+    """C5 at full size in training mode: the batch statistics over all 32768 tokens (what couples the tokens) against
+    float64 column statistics, the running-statistics update, and 32 sampled tokens through router, experts and MLP
+    against the oracle fed those statistics."""
+    from flash_moe.modules.flash_moe import FlashMoE, FlashMoEConfig
+    from flash_moe.ops.hip.flash_block import block_forward
+    from flash_moe.ops.hip.flash_router import router_forward
+
+    dtype, T, H, I, E, K, nk = torch.bfloat16, 32768, 2048, 8192, 262144, 128, 512
+    with torch.device("cuda"):
+        m = FlashMoE(FlashMoEConfig(H, I, "silu", E, K, True)).to(dtype)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.normal_(0.0, 0.02, generator=g)
+    m.train()
+    x = (torch.randn(8, 4096, H, device="cuda", generator=g) * 1.3 + 0.2).to(dtype)
+    tokens = x.view(T, H)
+    # statistics: mean and 1/sqrt(var + eps) the kernels normalise with, against float64
+    out = router_forward(tokens, m.router_gate.weight, m.router_norm, nk, K, True, return_logits32=True, return_stats=True)
+    logits, scores, indices, gates, logits32, stats = out
+    mean64, var64 = tokens.double().mean(0), tokens.double().var(0, unbiased=False)
+    torch.testing.assert_close(stats[:H].double(), mean64, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(stats[H:].double(), (var64 + 1e-5).rsqrt(), rtol=1e-5, atol=0)
+    assert int(m.router_norm.num_batches_tracked) == 1
+    torch.testing.assert_close(m.router_norm.running_mean.double(), 0.1 * mean64, rtol=2e-2, atol=2e-3)
+    torch.testing.assert_close(m.router_norm.running_var.double(), 0.9 + 0.1 * var64 * T / (T - 1), rtol=2e-2, atol=2e-3)
+    # the block in training mode: single call equals the staged routing on the same statistics
+    m.router_norm.reset_running_stats()
+    y, b_logits, b_idx, b_gates = block_forward(tokens, m.gate_proj.weight, m.up_proj.weight, m.down_proj.weight,
+                                                m.router_gate.weight, m.router_norm, m.down_embed.weight, m.up_embed.weight,
+                                                nk, K, True, return_routing=True)
+    assert torch.equal(b_idx, indices) and torch.equal(b_gates, gates) and torch.equal(b_logits, logits)
+    assert torch.isfinite(y).all()
+    # sampled tokens: gate logits from the normalised activations rounded to bf16, as a stand-alone batch-norm emits them
+    pick = torch.randperm(T, generator=torch.Generator().manual_seed(2))[:32].sort().values.cuda()
+    xs = tokens[pick]
+    q = ((xs.float() - stats[:H]) * stats[H:]).to(dtype)
+    ref32 = q.float() @ m.router_gate.weight.float().t()
+    assert rel_fro(logits32[pick], ref32) < 5e-4
+    lp = torch.log_softmax(logits32[pick].cpu().view(-1, 2, nk), dim=-1).transpose(0, 1).contiguous()
+    o_s, o_i = orc.router_topk(lp, nk, K + 1)
+    torch.testing.assert_close(scores[pick].cpu(), o_s[:, :K], rtol=0, atol=2e-6)
+    set_equal = (indices[pick].cpu().sort(-1).values == o_i[:, :K].sort(-1).values).all(-1)
+    assert (set_equal | ((o_s[:, K - 1] - o_s[:, K]).abs() < 2e-6)).all()
+    s_idx, s_gates = indices[pick], gates[pick]
+    rows, remap = torch.unique(s_idx, return_inverse=True)
+    wd_s, wu_s = m.down_embed.weight[rows].cpu().double(), m.up_embed.weight[rows].cpu().double()
+    e64 = orc.expert_forward(xs.cpu().double(), wd_s, wu_s, remap.cpu(), s_gates.cpu().double())
+    y64 = e64 + orc.mlp_forward(xs.cpu().double(), m.gate_proj.weight.cpu().double(), m.up_proj.weight.cpu().double(),
+                                m.down_proj.weight.cpu().double())
+    assert_output_close(y[pick], y64.to(dtype), dtype, "C5 train-mode block output vs float64 oracle on sampled tokens")
+
+
 def test_block_of_an_empty_batch():
     m, _ = build(128, 256, 1024, 8, False, torch.bfloat16)
     m.eval()
