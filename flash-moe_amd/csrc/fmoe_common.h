@@ -34,6 +34,14 @@ void clear_error();
         }                                                                              \
     } while (0)
 
+// What the launch geometry depends on: compute units, XCDs (workgroup ids are dealt round-robin over them, each has its
+// own L2) and the size of one L2, of the current device (fmoe_core.hip).
+struct ChipInfo {
+    int cus, xcds;
+    int64_t l2_bytes;
+};
+const ChipInfo& chip_info();
+
 // Top-k of the router taking raw fp32 gate outputs [T, 2*nk] (log-softmax per half is done inside); defined in
 // fmoe_router.hip, used by the fused router entry point.  gates has element type `gate_dtype`.  When `row_offsets`
 // is given, the byte offset id*row_bytes of each selected expert's table row is written next to its id.

@@ -252,10 +252,11 @@ __global__ __launch_bounds__(256) void expert_prepare_kernel(const int64_t* __re
     }
 }
 
-__device__ inline bool slice_of_block(int num_slices, int blocks_per_slice, int& slice, int& tb) {
+// Workgroup b runs on XCD b % xcds (ids are dealt round-robin): XCD x takes slices x, x + xcds, ...
+__device__ inline bool slice_of_block(int num_slices, int blocks_per_slice, int xcds, int& slice, int& tb) {
     const int b = (int)blockIdx.x;
-    const int j = b >> 3;
-    slice = (b & 7) + 8 * (j / blocks_per_slice);
+    const int j = b / xcds;
+    slice = b % xcds + xcds * (j / blocks_per_slice);
     tb = j % blocks_per_slice;
     return slice < num_slices;
 }
@@ -288,11 +289,11 @@ template <typename T, int CL>
 __global__ __launch_bounds__(256) void expert_scores_slice_kernel(
     const T* __restrict__ x, const T* __restrict__ down, uint32_t table_bytes, const uint32_t* __restrict__ off32,
     float* __restrict__ spart, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
-    int tokens_per_block) {
+    int tokens_per_block, int xcds) {
     constexpr int V = Elem<T>::kVec;
     constexpr int PPL = kWave / CL;                         // pairs per wave-wide load
     int slice, tb;
-    if (!slice_of_block(num_slices, blocks_per_slice, slice, tb)) return;
+    if (!slice_of_block(num_slices, blocks_per_slice, xcds, slice, tb)) return;
     const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
     const int c = lane & (CL - 1), pg = lane / CL;
     const int col = slice * (CL * V) + c * V;
@@ -377,11 +378,11 @@ template <typename T, int CL>
 __global__ __launch_bounds__(256) void expert_states_slice_kernel(
     const float* __restrict__ a, const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ off32,
     T* __restrict__ out, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
-    int tokens_per_block) {
+    int tokens_per_block, int xcds) {
     constexpr int V = Elem<T>::kVec;
     constexpr int PPL = kWave / CL;
     int slice, tb;
-    if (!slice_of_block(num_slices, blocks_per_slice, slice, tb)) return;
+    if (!slice_of_block(num_slices, blocks_per_slice, xcds, slice, tb)) return;
     const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
     const int c = lane & (CL - 1), pg = lane / CL;
     const int col = slice * (CL * V) + c * V;
@@ -425,7 +426,7 @@ __global__ __launch_bounds__(256) void expert_states_slice_kernel(
 }
 
 struct SlicePlan {
-    int chunk_lanes, num_slices, blocks_per_slice, tokens_per_block;
+    int chunk_lanes, num_slices, blocks_per_slice, tokens_per_block, xcds;
     unsigned grid;
     size_t off_idx32, off_a, off_spart, bytes;
 };
@@ -434,13 +435,15 @@ struct SlicePlan {
 // the offsets, coefficients and partial sums), 128 bytes beyond.
 SlicePlan plan_slices(int64_t T_, int H, int64_t E, int K, size_t elt) {
     SlicePlan p;
-    p.chunk_lanes = E * 256 <= (4ll << 20) ? 16 : 8;
+    const ChipInfo& chip = chip_info();
+    p.xcds = chip.xcds;
+    p.chunk_lanes = E * 256 <= chip.l2_bytes ? 16 : 8;
     const size_t chunk_bytes = (size_t)p.chunk_lanes * 16;
     p.num_slices = (int)((H * elt + chunk_bytes - 1) / chunk_bytes);
     const int64_t want = (T_ + 3) / 4;                       // at least one token per wave
     p.blocks_per_slice = (int)(want < 1024 ? want : 1024);   // 256 blocks of 4 waves fill one XCD; a few rounds of them
     p.tokens_per_block = (int)((T_ + p.blocks_per_slice - 1) / p.blocks_per_slice);
-    p.grid = (unsigned)(8 * p.blocks_per_slice * ((p.num_slices + 7) / 8));
+    p.grid = (unsigned)(p.xcds * p.blocks_per_slice * ((p.num_slices + p.xcds - 1) / p.xcds));
     const size_t pairs = (size_t)T_ * (size_t)K;
     p.off_idx32 = 0;
     p.off_a = round_up(p.off_idx32 + pairs * 4, 256);
@@ -457,11 +460,11 @@ int launch_slice_scores(const void* x, const void* table, const uint32_t* off32,
     if (p.chunk_lanes == 16)
         hipLaunchKernelGGL((expert_scores_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
                            (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
-                           p.tokens_per_block);
+                           p.tokens_per_block, p.xcds);
     else
         hipLaunchKernelGGL((expert_scores_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
                            (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
-                           p.tokens_per_block);
+                           p.tokens_per_block, p.xcds);
     FMOE_CHECK_LAUNCH("routed experts (slice scores)");
     return FMOE_OK;
 }
@@ -473,10 +476,10 @@ int launch_slice_states(const float* a, const void* table, const uint32_t* off32
     const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
     if (p.chunk_lanes == 16)
         hipLaunchKernelGGL((expert_states_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, a, (const T*)table,
-                           table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+                           table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block, p.xcds);
     else
         hipLaunchKernelGGL((expert_states_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, a, (const T*)table,
-                           table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block);
+                           table_bytes, off32, (T*)out, T_, H, K, p.num_slices, p.blocks_per_slice, p.tokens_per_block, p.xcds);
     FMOE_CHECK_LAUNCH("routed experts (slice states)");
     return FMOE_OK;
 }
@@ -563,7 +566,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const T* __restrict__ xb, uint32_t x_bytes, const T* __restrict__ down, uint32_t table_bytes,
     const uint32_t* __restrict__ entry, const uint32_t* __restrict__ expid, const int32_t* __restrict__ offsets,
     int64_t num_experts, float* __restrict__ spart, int64_t spart_stride, uint32_t row_bytes, int num_bands, int parts,
-    int blocks_per_unit) {
+    int blocks_per_unit, int xcds) {
     constexpr int G = kWave / CL, U = kBucketBatch;
     constexpr int kRun = 4 * G * kBucketChunk;                          // slots per workgroup iteration
     constexpr int kBand = CL * 16;
@@ -572,8 +575,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     static_assert(kBucketChunk == 8 * U && CL >= 8 && kRows <= 256, "lane c < 8 holds the entries of batch c");
     __shared__ __attribute__((aligned(16))) unsigned char rows[kBucketLdsBytes];
     const int b = (int)blockIdx.x;
-    const int unit = (b & 7) + 8 * ((b >> 3) / blocks_per_unit);       // XCD (b & 7) takes units x, x + 8, ...
-    const int tb = (b >> 3) % blocks_per_unit;
+    const int unit = b % xcds + xcds * ((b / xcds) / blocks_per_unit);  // XCD b % xcds takes units x, x + xcds, ...
+    const int tb = (b / xcds) % blocks_per_unit;
     if (unit >= num_bands * parts) return;
     const int band = unit % num_bands, part = unit / num_bands;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -780,13 +783,13 @@ template <typename T>
 __global__ __launch_bounds__(kSweepThreads) void expert_states_sweep_kernel(
     const T* __restrict__ up, uint32_t table_bytes, const uint32_t* __restrict__ entries, const float* __restrict__ coef,
     T* __restrict__ out, int64_t num_tokens, int64_t num_experts, int top_k, uint32_t row_bytes, int num_bands,
-    int token_blocks) {
+    int token_blocks, int xcds) {
     constexpr int CL = 8;
     static_assert(sizeof(T) == 2, "eight 16-bit columns per lane: a 128-byte band is 64 columns");
     __shared__ __attribute__((aligned(16))) float sums[kSweepWgTokens * 64];   // [512 tokens][64 columns]: 128 KiB
     const int b = (int)blockIdx.x;
-    const int band = (b & 7) + 8 * ((b >> 3) / token_blocks);           // XCD (b & 7) takes bands x, x + 8, ...
-    const int tb = (b >> 3) % token_blocks;
+    const int band = b % xcds + xcds * ((b / xcds) / token_blocks);     // XCD b % xcds takes bands x, x + xcds, ...
+    const int tb = (b / xcds) % token_blocks;
     if (band >= num_bands) return;
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int c = lane & (CL - 1), group = tid / CL;                    // lane group 0..127 of the workgroup
@@ -892,7 +895,7 @@ __global__ __launch_bounds__(kSweepThreads) void expert_states_sweep_kernel(
 }
 
 struct BucketedPlan {
-    int chunk_lanes, num_bands, parts, blocks_per_unit;
+    int chunk_lanes, num_bands, parts, blocks_per_unit, xcds;
     unsigned grid;
     size_t off_bucket, off_offsets, off_pairs, off_tok, off_exp, off_a, off_spart, off_xb, off_sweep_keys, off_sweep_coef, bytes;
     bool sweep;
@@ -907,17 +910,19 @@ bool sweep_possible(int64_t T_, int H, int64_t E, int K, size_t elt) {
 // Band width: as wide as lets the band of all tokens stay in one XCD's L2 (about 2 MiB of its 4), at least 128 bytes.
 BucketedPlan plan_bucketed(int64_t T_, int H, int64_t E, int K, size_t elt) {
     BucketedPlan p;
-    p.chunk_lanes = T_ * 512 <= (2ll << 20) ? 32 : (T_ * 256 <= (2ll << 20) ? 16 : 8);
+    const ChipInfo& chip = chip_info();
+    p.xcds = chip.xcds;
+    p.chunk_lanes = T_ * 512 <= chip.l2_bytes / 2 ? 32 : (T_ * 256 <= chip.l2_bytes / 2 ? 16 : 8);
     while (p.chunk_lanes > 8 && (H * elt) % ((size_t)p.chunk_lanes * 16) != 0) p.chunk_lanes /= 2;   // bands tile the row
     const size_t band_bytes = (size_t)p.chunk_lanes * 16;
     p.num_bands = (int)((H * elt + band_bytes - 1) / band_bytes);
-    p.parts = (p.num_bands < 8 && 8 % p.num_bands == 0) ? 8 / p.num_bands : 1;      // several XCDs share a band
+    p.parts = (p.num_bands < p.xcds && p.xcds % p.num_bands == 0) ? p.xcds / p.num_bands : 1;      // several XCDs share a band
     const int64_t pairs = T_ * K;
     const int64_t run_slots = 4 * (kWave / p.chunk_lanes) * kBucketChunk;
     const int64_t want = ((pairs + run_slots - 1) / run_slots + p.parts - 1) / p.parts;      // runs per part
     p.blocks_per_unit = (int)(want < 1 ? 1 : (want > 256 ? 256 : want));
     const int units = p.num_bands * p.parts;
-    p.grid = (unsigned)(8 * p.blocks_per_unit * ((units + 7) / 8));
+    p.grid = (unsigned)(p.xcds * p.blocks_per_unit * ((units + p.xcds - 1) / p.xcds));
     size_t o = 0;
     auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
     p.off_bucket = take(bucket_workspace_bytes(E));
@@ -975,7 +980,7 @@ int launch_expert_bucketed(int act, const void* x, const void* down, const void*
 #define FMOE_LAUNCH_BUCKETED(CLV)                                                                                          \
     hipLaunchKernelGGL((expert_scores_bucketed_kernel<T, CLV>), dim3(p.grid), dim3(256), 0, stream, (const T*)xb, x_bytes,  \
                        (const T*)down, table_bytes, (const uint32_t*)tokoff, (const uint32_t*)expoff, (const int32_t*)offsets, \
-                       E, spart, pairs, row_bytes, p.num_bands, p.parts, p.blocks_per_unit)
+                       E, spart, pairs, row_bytes, p.num_bands, p.parts, p.blocks_per_unit, p.xcds)
     if (p.chunk_lanes == 32) FMOE_LAUNCH_BUCKETED(32);
     else if (p.chunk_lanes == 16) FMOE_LAUNCH_BUCKETED(16);
     else FMOE_LAUNCH_BUCKETED(8);
@@ -999,10 +1004,10 @@ int launch_expert_bucketed(int act, const void* x, const void* down, const void*
             FMOE_CHECK_LAUNCH("fmoe_expert_forward(owner sort)");
             const int bands = (int)(row_bytes / 128);
             const int token_blocks = (int)((T_ + kSweepWgTokens - 1) / kSweepWgTokens);
-            const unsigned grid = (unsigned)(8 * token_blocks * ((bands + 7) / 8));
+            const unsigned grid = (unsigned)(p.xcds * token_blocks * ((bands + p.xcds - 1) / p.xcds));
             hipLaunchKernelGGL((expert_states_sweep_kernel<T>), dim3(grid), dim3(kSweepThreads), 0, stream, (const T*)up,
                                table_bytes, (const uint32_t*)keys, (const float*)coef, (T*)out, T_, E, K, row_bytes, bands,
-                               token_blocks);
+                               token_blocks, p.xcds);
             FMOE_CHECK_LAUNCH("fmoe_expert_forward(sweep)");
             return FMOE_OK;
         }
@@ -1010,10 +1015,10 @@ int launch_expert_bucketed(int act, const void* x, const void* down, const void*
     return launch_expert_rows_coef<T>(up, indices, a, T_, H, E, K, out, stream);
 }
 
-// A slice of the table must stay resident in one XCD's 4 MiB L2 next to the streaming traffic; with 128-byte
-// slices of up to 8 MiB the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
+// A slice of the table must stay resident in one XCD's L2 (4 MiB) next to the streaming traffic; with 128-byte
+// slices of up to twice the L2 the measured gather rate is still twice the fabric's.  Beyond that, and for problems with
 // too few pairs to pay for four launches, whole rows are gathered by the one-wave-per-token kernel.
-bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= (8ll << 20) && T_ * K >= (1ll << 16); }
+bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= 2 * chip_info().l2_bytes && T_ * K >= (1ll << 16); }
 // rows are addressed with 32-bit byte offsets below kBadOffset
 bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
 

@@ -28,10 +28,10 @@ __device__ inline int swizzled_offset(int row, int chunk) { return row * kTileK 
 
 // Map the linear workgroup id to a tile so that each XCD gets a contiguous run of the tile order, and the tile order
 // walks 8 tile-rows at a time (compact patches share A and B tiles in the XCD's L2).
-__device__ inline void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ inline void tile_of_block(int tiles_m, int tiles_n, int xcds, int& tm, int& tn) {
     const int nb = (int)gridDim.x;
     int t = (int)blockIdx.x;
-    if ((nb & 7) == 0) t = (t & 7) * (nb >> 3) + (t >> 3);
+    if (nb % xcds == 0) t = (t % xcds) * (nb / xcds) + t / xcds;
     constexpr int GM = 8;
     const int width = GM * tiles_n;
     const int group = t / width;

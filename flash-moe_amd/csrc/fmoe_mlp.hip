@@ -34,7 +34,7 @@ template <bool B> struct Flag { static constexpr bool value = B; };
 template <typename T, int BM, int BN, int EPI>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
     const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
-    const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n) {
+    const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n, int xcds) {
     using Frag = typename Mfma32<T>::Frag;
     constexpr int WM = BM / 2, WN = BN / 2;        // per-wave tile
     constexpr int MF = WM / 32, NF = WN / 32;      // 32x32 fragments per wave
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
     __shared__ __attribute__((aligned(16))) T Bs[BN * BK];
 
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n, tm, tn);
+    tile_of_block(tiles_m, tiles_n, xcds, tm, tn);
     const int m0 = tm * BM;
     const int n0 = tn * BN_OUT;
 
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
-    const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n) {
+    const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n, int xcds) {
     using Frag = typename Mfma32<T>::Frag;
     constexpr int NWAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MF = WM / 32, NF = WN / 32;
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     // The workgroup is persistent: it takes tiles t, t + gridDim.x, ...  Each XCD (workgroup id mod 8) gets a contiguous
     // run of the tile order, walked 8 tile-rows at a time so that a compact patch shares A and B tiles in the XCD's L2.
     auto set_tile = [&](int t) {
-        if ((num_tiles & 7) == 0) t = (t & 7) * (num_tiles >> 3) + (t >> 3);
+        if (num_tiles % xcds == 0) t = (t % xcds) * (num_tiles / xcds) + t / xcds;
         constexpr int GM = 8;
         const int width = GM * tiles_n, group = t / width, first_m = group * GM;
         const int gsz = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
@@ -504,7 +504,7 @@ void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, 
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_OUT - 1) / BN_OUT;
     hipLaunchKernelGGL((gemm_nt_kernel<T, BM, BN, EPI>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), 0,
-                       stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
+                       stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n, chip_info().xcds);
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
@@ -515,19 +515,20 @@ void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int
     constexpr int kStageBytes = (BM + BN) * BKT * (int)sizeof(T) * NSTAGE;
     constexpr int kPerCu = (160 * 1024 / kStageBytes) < 1 ? 1 : ((160 * 1024 / kStageBytes) > 2 ? 2 : (160 * 1024 / kStageBytes));
     const int total = tiles_m * tiles_n;
-    const int resident = 256 * kPerCu;
+    const ChipInfo& chip = chip_info();
+    const int resident = chip.cus * kPerCu;
     const int grid = total < resident ? total : resident;
     hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI, PF>), dim3((unsigned)grid),
-                       dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n);
+                       dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n, chip.xcds);
 }
 
-// Tile choice: 256-wide tiles (8 waves, two per SIMD) halve the L2 -> LDS traffic per MFMA but need >= 256 of them to
+// Tile choice: 256-wide tiles (8 waves, two per SIMD) halve the L2 -> LDS traffic per MFMA but need one per CU to
 // occupy the chip; otherwise 128x128 tiles of 4 waves, which read a whole k-tile of fragments ahead (PF = 3): one
 // workgroup per CU with four stages in flight when every tile gets a CU of its own, two per CU with two stages else.
 template <typename T, int EPI>
 void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, int64_t tiles,
                         hipStream_t stream) {
-    if (tiles <= 256) launch_gemm_dma<T, 128, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+    if (tiles <= chip_info().cus) launch_gemm_dma<T, 128, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
     else launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
 }
 
@@ -535,7 +536,7 @@ void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, 
 // every CU a tile.  N_OUT: output columns of a tile.
 template <typename T, int EPI>
 void launch_narrow_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
-    if (EPI == kEpiPlain && (int64_t)((M + 63) / 64) * (N / 128) < 256 && N % 64 == 0)
+    if (EPI == kEpiPlain && (int64_t)((M + 63) / 64) * (N / 128) < chip_info().cus && N % 64 == 0)
         launch_gemm_dma<T, 64, 64, 2, 2, 64, 4, kEpiPlain, 3>(A, B0, B1, C, R, M, N, K, stream);
     else
         launch_gemm_dma<T, 64, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
@@ -545,9 +546,9 @@ template <typename T>
 int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
     const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu, *S = (const T*)saved;
     const bool k_ok = H % 64 == 0;
-    if (k_ok && I % 128 == 0 && (int64_t)((M + 255) / 256) * (I / 128) >= 256)
+    if (k_ok && I % 128 == 0 && (int64_t)((M + 255) / 256) * (I / 128) >= chip_info().cus)
         launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, S, M, I, H, stream);
-    else if (k_ok && I % 64 == 0 && (int64_t)((M + 127) / 128) * (I / 64) >= 256)
+    else if (k_ok && I % 64 == 0 && (int64_t)((M + 127) / 128) * (I / 64) >= chip_info().cus)
         launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, (int64_t)((M + 127) / 128) * (I / 64), stream);
     else if (k_ok && I % 64 == 0)
         launch_narrow_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
@@ -561,9 +562,9 @@ template <typename T>
 int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
     const T *A = (const T*)h, *W = (const T*)wd, *R = (const T*)residual;
     const bool k_ok = I % 64 == 0;
-    if (k_ok && H % 256 == 0 && (int64_t)((M + 255) / 256) * (H / 256) >= 256)
+    if (k_ok && H % 256 == 0 && (int64_t)((M + 255) / 256) * (H / 256) >= chip_info().cus)
         launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiPlain, 1>(A, W, nullptr, (T*)out, R, M, H, I, stream);
-    else if (k_ok && H % 128 == 0 && (int64_t)((M + 127) / 128) * (H / 128) >= 256)
+    else if (k_ok && H % 128 == 0 && (int64_t)((M + 127) / 128) * (H / 128) >= chip_info().cus)
         launch_small_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, (int64_t)((M + 127) / 128) * (H / 128), stream);
     else if (k_ok && H % 128 == 0)
         launch_narrow_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);

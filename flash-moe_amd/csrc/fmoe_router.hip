@@ -289,7 +289,7 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
                   int norm, uint32_t* row_offsets, uint32_t row_bytes, hipStream_t stream) {
     const int num_cand = count_candidates(K);
     const int64_t blocks_needed = (T_ + kRouterWaves - 1) / kRouterWaves;
-    const int64_t max_blocks = 256 * 8;   // a few resident blocks per CU; the kernel loops over tokens
+    const int64_t max_blocks = (int64_t)chip_info().cus * 8;   // a few resident blocks per CU; the kernel loops over tokens
     const dim3 grid((unsigned)(blocks_needed < max_blocks ? blocks_needed : max_blocks));
     const dim3 block(kRouterWaves * kWave);
 #define FMOE_LAUNCH_ROUTER(R)                                                                                      \

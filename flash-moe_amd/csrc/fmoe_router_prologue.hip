@@ -252,7 +252,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const float* __restrict__ mean_rstd, float* __restrict__ logits32,
                                                           T* __restrict__ logits, int M, int N, int K_full, int tiles_m,
-                                                          int tiles_n, int split) {
+                                                          int tiles_n, int split, int xcds) {
     using Frag = typename Mfma32<T>::Frag;
     constexpr int BM = 64, BN = 64, CH = 2;   // CH = 16-byte packets per thread per tile and operand
     constexpr int D = kGatePrefetch;
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ 
     __shared__ __attribute__((aligned(16))) T Bs[BN * kTileK];
     extern __shared__ __attribute__((aligned(16))) float stats[];   // [2][Kpad]: mean, rstd
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n, tm, tn);
+    tile_of_block(tiles_m, tiles_n, xcds, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -824,11 +824,11 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
         if (dtype == FMOE_BF16)
             hipLaunchKernelGGL((router_gate_kernel<bf16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
                                (const bf16_t*)x, (const bf16_t*)gate_w, (const float*)mean_rstd, logits32,
-                               (bf16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query);
+                               (bf16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query, chip_info().xcds);
         else
             hipLaunchKernelGGL((router_gate_kernel<f16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
                                (const f16_t*)x, (const f16_t*)gate_w, (const float*)mean_rstd, logits32,
-                               (f16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query);
+                               (f16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query, chip_info().xcds);
     }
     FMOE_CHECK_LAUNCH("fmoe_router_forward(gate)");
     if (top_k == 0) return FMOE_OK;
