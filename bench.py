@@ -12,8 +12,14 @@ that is already resident in HBM.  The last line printed is one JSON object:
   roofline       the slowest C-ABI call of the block (its kernels are named in `launches`) against the roofline
                  that bounds it; rooflines_all has every call
   expert_c3      the routed-expert kernel alone on its own benchmark shape (16384 tokens), as HBM GB/s
+  router_c2      the routing stage alone on the router benchmark shape: module semantics (every half scores the full
+                 query) and the configuration as worded (two sub-key tables on the two halves of the query)
+  block_c5       the largest block (32768 tokens, 262144 experts), with its stages and the expert op's roofline entry
   cpu_baseline   the CPU restatement of the reference's eager path (oracle/) on the same block, timed on
-                 this machine's host cores
+                 this machine's host cores; cpu_baseline_c1 / cpu_baseline_c4_fp32: the reference's own CPU
+                 configuration (fp32, 512 tokens) and the README block in fp32
+  `traffic` figures are fabric-side bytes per launch (L2 misses, whether the Infinity Cache or HBM serves them) from
+  rocprofv3 FETCH_SIZE / WRITE_SIZE runs kept under profiles/; the calibration is stated in traffic_source.
 
 Only one GPU is used; --gpus N with N > 1 exits with a message.
 """
@@ -35,6 +41,7 @@ for p in (ROOT, os.path.join(ROOT, "flash-moe_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 
+C1 = dict(batch=1, seq=512, hidden=256, inter=1024, experts=1024, top_k=16, norm=False)
 C4 = dict(batch=1, seq=4096, hidden=1024, inter=4096, experts=16384, top_k=64, norm=False)
 C3 = dict(tokens=16384, hidden=1024, experts=16384, top_k=64)
 C2 = dict(tokens=8192, hidden=1024, keys=128, top_k=64)
@@ -149,7 +156,8 @@ def stage_kernels(m, x):
     touched = int(torch.unique(indices).numel())
     elt = x.element_size()
     work = {
-        "router_forward": dict(bound="hbm", bytes=T * H * elt + 2 * nk * H * elt + T * 2 * nk * (elt + 4) + T * K * (4 + 8 + elt)),
+        "router_forward": dict(bound="hbm", bytes=T * H * elt + 2 * nk * H * elt + T * 2 * nk * (elt + 4) + T * K * (4 + 8 + elt),
+                               flops=2 * T * H * 2 * nk),
         "router_topk": dict(bound="hbm", bytes=2 * T * nk * 4 + T * K * (4 + 8 + 4)),
         "expert": dict(bound="hbm", bytes=expert_bytes(T, H, K, touched, elt), touched_experts=touched),
         "mlp_gate_up": dict(bound="mfma", flops=2 * T * H * 2 * I),
@@ -164,25 +172,39 @@ LAUNCHES = {
     "router_forward": ["bn_partial_kernel", "bn_finalize_kernel", "router_gate_kernel", "router_topk_kernel"],
     "router_topk": ["router_topk_kernel"],
     "expert": ["expert_prepare_kernel", "expert_scores_slice_kernel", "expert_gate_kernel", "expert_states_slice_kernel"],
+    "expert_c5": ["bucket_clear_kernel", "bucket_histogram_kernel", "bucket_scan_kernel", "bucket_fill_kernel",
+                  "expert_band_copy_kernel", "expert_scores_bucketed_kernel", "expert_gate_sorted_kernel",
+                  "expert_owner_sort_kernel", "expert_states_sweep_kernel"],
     "mlp_gate_up": ["gemm_dma_kernel<256x256 tiles, SwiGLU epilogue>"],
     "mlp_down": ["gemm_dma_kernel<128x128 tiles, residual epilogue>"],
 }
 
 
-def roofline_entry(name, ms, w, traffic):
+def roofline_entry(name, ms, w, traffic, launches=None):
     if w["bound"] == "hbm":
         achieved = w["bytes"] / (ms * 1e-3) / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
     else:
         achieved = w["flops"] / (ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
-    return dict(kernel=name, launches=LAUNCHES.get(name, [name]), bound=w["bound"], achieved=round(achieved, 2), peak=peak,
-                unit=unit, frac=round(achieved / peak, 4), avg_launch_us=round(ms * 1e3, 2),
-                algorithmic=w.get("bytes", w.get("flops")), traffic=traffic)
+    entry = dict(kernel=name, launches=LAUNCHES.get(launches or name, [name]), bound=w["bound"], achieved=round(achieved, 2),
+                 peak=peak, unit=unit, frac=round(achieved / peak, 4), avg_launch_us=round(ms * 1e3, 2),
+                 algorithmic=w.get("bytes", w.get("flops")), traffic=traffic)
+    if w["bound"] == "hbm" and "flops" in w:
+        # a contraction below the MFMA ridge: the matrix-core fraction next to the binding (HBM) one
+        tf = w["flops"] / (ms * 1e-3) / 1e12
+        entry["mfma_TFLOPs"] = round(tf, 2)
+        entry["mfma_frac"] = round(tf / MFMA_BF16_PEAK_TFLOPS, 4)
+    return entry
+
+
+TRAFFIC_SOURCE = ("fabric-side bytes per launch (L2 misses, served by the Infinity Cache or HBM) = 2.000 x FETCH_SIZE + 1.000 x "
+                  "WRITE_SIZE in KiB per dispatch from two rocprofv3 --pmc runs; the factors are what the same counters read "
+                  "for a 256 MiB device copy (profiles/hbm_traffic_counters.txt)")
 
 
 def measured_traffic(kernel, workload):
-    """HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, if a summary is committed."""
+    """Fabric-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, if a summary is committed."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
@@ -263,14 +285,36 @@ def bench_router_c2(dtype, iters):
         if rc:
             raise RuntimeError(L.fmoe_last_error().decode())
 
-    ms_fused, ms_topk = event_time_ms(fused, iters), event_time_ms(topk, iters)
+    # the configuration as worded: two sub-key tables [nk, H/2], each on its own half of the query
+    w_split = (torch.randn(2 * nk, H // 2, generator=g) * 0.02).to(dtype).cuda()
+
+    def split():
+        rc = L.fmoe_router_forward_split(x.data_ptr(), w_split.data_ptr(), None, None, None, code, 1, 0.1, 1e-5, T, H, nk, K,
+                                         code, 0, logits.data_ptr(), logits32.data_ptr(), scores.data_ptr(),
+                                         indices.data_ptr(), gates.data_ptr(), ws.data_ptr(), ws_bytes, stream())
+        if rc:
+            raise RuntimeError(L.fmoe_last_error().decode())
+
+    ms_fused, ms_topk, ms_split = event_time_ms(fused, iters), event_time_ms(topk, iters), event_time_ms(split, iters)
     elt = x.element_size()
     nbytes = T * H * elt + 2 * nk * H * elt + T * 2 * nk * elt + T * K * (elt + 8)
+    nbytes_split = nbytes - nk * H * elt
+    flops, flops_split = 2 * T * H * 2 * nk, T * H * 2 * nk
     return dict(workload=f"router only: bf16, {T} tokens, hidden {H}, 2x{nk} keys, top-{K}, train-mode batch norm",
                 fused_us=round(ms_fused * 1e3, 2), topk_only_us=round(ms_topk * 1e3, 2),
                 tokens_per_s=round(T / (ms_fused * 1e-3)), algorithmic_bytes=nbytes,
                 achieved_GBps=round(nbytes / (ms_fused * 1e-3) / 1e9, 1), peak_GBps=HBM_PEAK_GBS,
-                gemm_TFLOPs=round(2 * T * H * 2 * nk / (ms_fused * 1e-3) / 1e12, 2))
+                frac=round(nbytes / (ms_fused * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                gemm_TFLOPs=round(flops / (ms_fused * 1e-3) / 1e12, 2),
+                mfma_frac=round(flops / (ms_fused * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                as_worded=dict(workload=f"two sub-key tables {nk} x {H // 2}, each on its own half of the {H}-wide query "
+                                        "(fmoe_router_forward_split)",
+                               fused_us=round(ms_split * 1e3, 2), tokens_per_s=round(T / (ms_split * 1e-3)),
+                               algorithmic_bytes=nbytes_split,
+                               achieved_GBps=round(nbytes_split / (ms_split * 1e-3) / 1e9, 1),
+                               frac=round(nbytes_split / (ms_split * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                               gemm_TFLOPs=round(flops_split / (ms_split * 1e-3) / 1e12, 2),
+                               mfma_frac=round(flops_split / (ms_split * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)))
 
 
 def bench_block_c5(dtype, iters):
@@ -290,9 +334,17 @@ def bench_block_c5(dtype, iters):
     T = cfg["batch"] * cfg["seq"]
     with torch.no_grad():
         ms = event_time_ms(lambda: m(x), iters, warmup=2)
+        fns, work, keep = stage_kernels(m, x)
+        times = {n: event_time_ms(fn, iters, warmup=2) for n, fn in fns.items()}
+    expert = roofline_entry("expert", times["expert"], work["expert"], measured_traffic("expert", "c5"), launches="expert_c5")
+    expert["touched_experts"] = work["expert"]["touched_experts"]
+    del keep, fns
     return dict(workload=f"C5 full block: bf16, {T} tokens, hidden {cfg['hidden']}, intermediate {cfg['inter']}, "
                          f"{cfg['experts']} experts, top-{cfg['top_k']}, norm_topk_prob True, train-mode batch norm",
-                ms_per_step=round(ms, 3), tokens_per_s=round(T / (ms * 1e-3)))
+                ms_per_step=round(ms, 3), tokens_per_s=round(T / (ms * 1e-3)),
+                stages_us={n: round(t * 1e3, 1) for n, t in times.items()},
+                expert=expert,
+                mlp_TFLOPs=round(6 * T * cfg["hidden"] * cfg["inter"] / ((times["mlp_gate_up"] + times["mlp_down"]) * 1e-3) / 1e12, 1))
 
 
 def bench_backward_c4(dtype, iters):
@@ -319,7 +371,18 @@ def bench_backward_c4(dtype, iters):
                 forward_autograd_ms=round(ms_fwd, 3))
 
 
-def cpu_baseline(cfg, dtype, budget_s=20.0):
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(cfg, dtype, budget_s=20.0, label="C4"):
     """The oracle's block forward on the same workload, on the host cores (checker timed as a baseline)."""
     import torch
 
@@ -341,8 +404,9 @@ def cpu_baseline(cfg, dtype, budget_s=20.0):
                 break
     med = statistics.median(times)
     return dict(value=round(T / med, 1), unit="tokens/s", cores=threads, kind="port",
-                sample=f"whole C4 batch ({T} tokens, {str(dtype).replace('torch.', '')}), median of {len(times)} "
-                       f"forward passes of the torch CPU restatement of FlashMoE_Pytorch.forward, {threads} threads",
+                sample=f"whole {label} batch ({T} tokens, {str(dtype).replace('torch.', '')}), median of {len(times)} "
+                       f"forward passes of the torch CPU restatement of FlashMoE_Pytorch.forward, {threads} threads "
+                       f"of {os.cpu_count()} logical CPUs ({cpu_model()})",
                 ms_per_step=round(med * 1e3, 2))
 
 
@@ -355,6 +419,7 @@ def main():
     ap.add_argument("--no-c3", action="store_true")
     ap.add_argument("--only-c3", action="store_true", help="run only the routed-expert kernel on its own shape (for profiling)")
     ap.add_argument("--only-backward", action="store_true", help="run only forward + backward of the C4 block (for profiling)")
+    ap.add_argument("--only-c5", action="store_true", help="run only the largest block (C5) and its stages (for profiling)")
     ap.add_argument("--no-extras", action="store_true", help="skip the router-only (C2) and largest-block (C5) side measurements")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 256 MiB device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
@@ -386,6 +451,13 @@ def main():
         log("expert C3:", res)
         print(json.dumps({"metric": "expert kernel HBM GB/s", "value": res["achieved_GBps"], "unit": "GB/s", "n_gpus": 1,
                           "steps": args.steps, "warmup": args.warmup, "expert_c3": res}), flush=True)
+        return
+    if args.only_c5:
+        res = bench_block_c5(dtype, max(3, min(10, args.steps)))
+        log("block C5:", res)
+        print(json.dumps({"metric": "FlashMoE fwd tokens/s (h2048, 256K experts, top-128)", "value": res["tokens_per_s"],
+                          "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "block_c5": res}),
+              flush=True)
         return
     if args.only_backward:
         res = bench_backward_c4(dtype, max(5, min(20, args.steps)))
@@ -441,7 +513,11 @@ def main():
                    "top_k": C4["top_k"]},
         "roofline": rooflines[dominant],
         "stages_us": stages,
+        # the block's own launches: the stages without the stand-alone top-k and without the expert op's id -> offset
+        # pass (inside the block the router writes the offsets); what is left of ms_per_step is launch gaps
+        "stages_sum_us": round(sum(v for k, v in stages.items() if k != "router_topk"), 2),
         "rooflines_all": rooflines,
+        "traffic_source": TRAFFIC_SOURCE,
     }
     if not args.no_c3:
         result["expert_c3"] = bench_expert_c3(dtype, max(10, min(50, args.steps)))
@@ -459,8 +535,13 @@ def main():
         log("backward C4:", result["backward_c4"])
         torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(C4, dtype)
+        result["cpu_baseline"] = cpu_baseline(C4, dtype, budget_s=12.0)
         log("cpu baseline:", result["cpu_baseline"])
+        # the reference's own CPU configuration (fp32, 512 tokens, 1024 experts, top-16) and the README block in fp32
+        result["cpu_baseline_c1"] = cpu_baseline(C1, torch.float32, budget_s=4.0, label="C1")
+        log("cpu baseline C1:", result["cpu_baseline_c1"])
+        result["cpu_baseline_c4_fp32"] = cpu_baseline(C4, torch.float32, budget_s=6.0)
+        log("cpu baseline C4 fp32:", result["cpu_baseline_c4_fp32"])
     print(json.dumps(result), flush=True)
 
 
