@@ -278,6 +278,174 @@ __global__ __launch_bounds__(kRouterWaves* kWave) __attribute__((amdgpu_waves_pe
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// Selection by threshold (num_keys <= 64*RH, candidates <= 64*RC): the same result as the group scan above, for the
+// sizes where a whole list fits the wave's registers (R keys per lane).
+//   1. tau = K-th largest score of the list, found bit by bit from the top: the largest value with at least K scores
+//      >= it (per bit one compare per register, the counts come from the ballots on the scalar unit);
+//   2. the keys above tau, then keys equal to tau in list order until K are taken, go to K slots in LDS (positions from
+//      ballot prefix counts);
+//   3. one bitonic sort of the KP slots on the 64-bit keys.
+// List order is key index order for a half (position p = r*64 + lane), so ties at the cut go to the lowest index there;
+// among candidate sums tied at the cut the earlier candidate (lower rank in half 0) is taken.
+// ------------------------------------------------------------------------------------------------------------
+template <int R>
+__device__ inline uint32_t kth_largest_score(const uint64_t (&key)[R], int k) {
+    uint32_t tau = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t trial = tau | (1u << bit);
+        int count = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            count += __builtin_popcountll(__builtin_amdgcn_ballot_w64((uint32_t)(key[r] >> 32) >= trial));
+        tau = count >= k ? trial : tau;
+    }
+    return tau;
+}
+
+__device__ inline int lanes_below(uint64_t mask) {
+    return (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+// slots: KP wave-private LDS entries.  Unused list entries hold key 0 (below every score).
+template <int R, int RK>
+__device__ inline void select_topk_sorted(const uint64_t (&key)[R], int k, uint64_t* slots, uint64_t (&best)[RK], int lane) {
+    constexpr int KP = RK * kWave;
+    const uint32_t tau = kth_largest_score<R>(key, k);
+    int base = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const bool above = (uint32_t)(key[r] >> 32) > tau;
+        const uint64_t m = __builtin_amdgcn_ballot_w64(above);
+        if (above) slots[base + lanes_below(m)] = key[r];
+        base += __builtin_popcountll(m);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const bool equal = (uint32_t)(key[r] >> 32) == tau;
+        const uint64_t m = __builtin_amdgcn_ballot_w64(equal);
+        const int pos = base + lanes_below(m);
+        if (equal && pos < k) slots[pos] = key[r];
+        base += __builtin_popcountll(m);
+    }
+    for (int p = k + lane; p < KP; p += kWave) slots[p] = 0ull;
+    __builtin_amdgcn_wave_barrier();      // LDS operations of one wave complete in order; keep the compiler from moving them
+#pragma unroll
+    for (int r = 0; r < RK; ++r) best[r] = slots[lane * RK + r];
+    __builtin_amdgcn_wave_barrier();
+    bitonic_sort<RK, true>(best, lane);
+}
+
+template <typename T, typename TG, int RK, int RH, int RC, bool FROM_LOGITS>
+__global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
+    const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
+    int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets,
+    uint32_t row_bytes) {
+    constexpr int KP = RK * kWave;
+    __shared__ uint16_t cand[RC * kWave];
+    __shared__ float half_score[kRouterWaves][2][KP];
+    __shared__ uint32_t half_index[kRouterWaves][2][KP];
+    __shared__ uint64_t slot[kRouterWaves][KP];
+
+    // candidate table, as in router_topk_kernel
+    {
+        uint32_t* row_len = &half_index[0][0][0];
+        for (int i = threadIdx.x; i < top_k; i += blockDim.x) row_len[i] = (uint32_t)(top_k / (i + 1));
+        __syncthreads();
+        for (int i = threadIdx.x; i < top_k; i += blockDim.x) {
+            int off = 0;
+            for (int q = 0; q < i; ++q) off += (int)row_len[q];
+            const int n = (int)row_len[i];
+            for (int j = 0; j < n; ++j) cand[off + j] = (uint16_t)(i | (j << 8));
+        }
+        __syncthreads();
+    }
+
+    const int lane = lane_id();
+    const int wave = (int)(threadIdx.x >> 6);
+    const int64_t waves_total = (int64_t)gridDim.x * kRouterWaves;
+    const int64_t rounds = (num_tokens + waves_total - 1) / waves_total;
+
+    for (int64_t round = 0; round < rounds; ++round) {
+        const int64_t token = round * waves_total + (int64_t)blockIdx.x * kRouterWaves + wave;
+        if (token >= num_tokens) continue;           // nothing below synchronises across waves
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const T* row = FROM_LOGITS ? lp + (token * 2 + h) * nk : lp + ((int64_t)h * num_tokens + token) * nk;
+            float v[RH];
+#pragma unroll
+            for (int r = 0; r < RH; ++r) {
+                const int p = r * kWave + lane;
+                v[r] = p < nk ? Elem<T>::to_f32(row[p]) : 0.0f;
+            }
+            float shift = 0.0f, lse = 0.0f;
+            if (FROM_LOGITS) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int r = 0; r < RH; ++r)
+                    if (r * kWave + lane < nk) mx = fmaxf(mx, v[r]);
+                mx = wave_max(mx);
+                float se = 0.0f;
+#pragma unroll
+                for (int r = 0; r < RH; ++r)
+                    if (r * kWave + lane < nk) se += expf(v[r] - mx);
+                shift = mx;
+                lse = logf(wave_sum(se));
+            }
+            uint64_t key[RH];
+#pragma unroll
+            for (int r = 0; r < RH; ++r) {
+                const int p = r * kWave + lane;
+                key[r] = p < nk ? make_key(FROM_LOGITS ? (v[r] - shift) - lse : v[r], (uint32_t)p) : 0ull;
+            }
+            uint64_t best[RK];
+            // every rank up to KP is looked up by the candidates (entries past nk stay key 0)
+            select_topk_sorted<RH, RK>(key, nk < KP ? nk : KP, slot[wave], best, lane);
+#pragma unroll
+            for (int r = 0; r < RK; ++r) {
+                half_score[wave][h][lane * RK + r] = key_score(best[r]);
+                half_index[wave][h][lane * RK + r] = key_index(best[r]);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        uint64_t ckey[RC];
+#pragma unroll
+        for (int r = 0; r < RC; ++r) {
+            const int c = r * kWave + lane;
+            ckey[r] = 0ull;
+            if (c < num_cand) {
+                const int ij = cand[c];
+                const int i = ij & 0xff, j = ij >> 8;
+                const float s = round_through<T>(half_score[wave][0][i] + half_score[wave][1][j]);
+                const uint32_t flat = half_index[wave][0][i] * (uint32_t)nk + half_index[wave][1][j];
+                ckey[r] = make_key(s, flat);
+            }
+        }
+        uint64_t best[RK];
+        select_topk_sorted<RC, RK>(ckey, top_k, slot[wave], best, lane);
+        float e[RK];
+        float total = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RK; ++r) {
+            const int p = lane * RK + r;
+            e[r] = p < top_k ? expf(key_score(best[r])) : 0.0f;
+            total += e[r];
+        }
+        if (gates != nullptr && norm_topk_prob) total = wave_sum(total);
+#pragma unroll
+        for (int r = 0; r < RK; ++r) {
+            const int p = lane * RK + r;
+            if (p < top_k) {
+                const int64_t o = token * top_k + p;
+                scores[o] = Elem<T>::from_f32(key_score(best[r]));
+                indices[o] = (int64_t)key_index(best[r]);
+                if (row_offsets != nullptr) row_offsets[o] = key_index(best[r]) * row_bytes;
+                if (gates != nullptr) gates[o] = Elem<TG>::from_f32(norm_topk_prob ? e[r] / total : e[r]);
+            }
+        }
+    }
+}
+
 int count_candidates(int top_k) {
     int n = 0;
     for (int i = 1; i <= top_k; ++i) n += top_k / i;
@@ -292,6 +460,23 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
     const int64_t max_blocks = (int64_t)chip_info().cus * 8;   // a few resident blocks per CU; the kernel loops over tokens
     const dim3 grid((unsigned)(blocks_needed < max_blocks ? blocks_needed : max_blocks));
     const dim3 block(kRouterWaves * kWave);
+    // lists that fit the registers of a wave take the threshold selection
+#define FMOE_LAUNCH_SELECT(RK_, RH_, RC_)                                                                              \
+    hipLaunchKernelGGL((router_select_kernel<T, TG, RK_, RH_, RC_, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, \
+                       T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes)
+    if (K <= 64 && nk <= 512) {
+        if (nk <= 128) FMOE_LAUNCH_SELECT(1, 2, 5);
+        else FMOE_LAUNCH_SELECT(1, 8, 5);
+        FMOE_CHECK_LAUNCH("fmoe_router_topk");
+        return FMOE_OK;
+    }
+    if (K <= 128 && nk <= 512) {
+        if (nk <= 128) FMOE_LAUNCH_SELECT(2, 2, 11);
+        else FMOE_LAUNCH_SELECT(2, 8, 11);
+        FMOE_CHECK_LAUNCH("fmoe_router_topk");
+        return FMOE_OK;
+    }
+#undef FMOE_LAUNCH_SELECT
 #define FMOE_LAUNCH_ROUTER(R)                                                                                      \
     hipLaunchKernelGGL((router_topk_kernel<T, TG, R, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, T_, nk, K, \
                        num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes)

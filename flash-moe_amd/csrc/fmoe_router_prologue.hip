@@ -3,15 +3,19 @@
 //   logits = q Wr^T     [T, 2*nk]
 //   log-softmax per half, top-k over the pair sums, exp / renormalise   (router_topk_kernel, logits-input mode)
 //
-// Launches:
-//   bn_partial_kernel   per (row block, 512-column strip): shifted sums -> (mean, M2, n) of the block      [training]
-//   bn_finalize_kernel  per column: Chan's parallel combination of the blocks -> mean, 1/sqrt(var+eps);
-//                       running-statistics update (momentum, unbiased variance) and batch counter
-//   router_gate_kernel  MFMA GEMM whose A tile is normalised while it is staged: (x - mean) * rstd is rounded to the
-//                       activation dtype exactly as a stand-alone batch-norm would emit it, then multiplied with the
-//                       gate weights with fp32 accumulation; writes the logits in fp32 (for the routing) and in the
-//                       activation dtype (the tensor the module returns)
-//   router_topk_kernel  (fmoe_router.hip)
+// Launches, 16-bit activations (three in training mode, two in evaluation mode):
+//   bn_block_stats_kernel  per (row block, 128-byte column strip): shifted sums -> (mean, M2) of the block   [training]
+//   router_gate_kernel     MFMA GEMM.  Its prologue combines the (at most 16) row blocks per column (Chan's parallel
+//                          formula) into mean and 1/sqrt(var+eps) - or takes the running statistics - for the columns
+//                          it multiplies, and a few workgroups also store them and update the running statistics
+//                          (momentum, unbiased variance) and the batch counter.  The A tile is normalised while it is
+//                          staged: (x - mean) * rstd is rounded to the activation dtype exactly as a stand-alone
+//                          batch-norm would emit it, then multiplied with the gate weights with fp32 accumulation;
+//                          writes the logits in fp32 (for the routing) and in the activation dtype (the tensor the
+//                          module returns)
+//   router_topk_kernel     (fmoe_router.hip)
+// fp32 activations (a parity configuration, not tuned): bn_partial_kernel per (row block, 512-column strip),
+// bn_finalize_kernel per column, router_gate_f32_kernel, router_topk_kernel.
 #include <math.h>
 
 #include <mutex>
@@ -138,6 +142,121 @@ __global__ __launch_bounds__(kStatsThreads) void bn_partial_kernel(const T* __re
     }
 }
 
+// Statistics for the gate kernel's own prologue: few, tall row blocks, so that a gate workgroup can combine them itself.
+// Block (rb, strip): rows [rb*rows_per_block, ...), 8*V columns (one 128-byte line per row for 16-bit elements).  A wave's
+// load covers 8 rows (lanes 8 apart hold the same columns); the 4 waves take rows 8 apart.  Sums are relative to the
+// block's first row, as in bn_partial_kernel.  partial: [row_blocks][2][H] = (mean, M2); the row count of a block follows
+// from the geometry.
+constexpr int kFoldMaxRowBlocks = 16;
+template <typename T>
+__global__ __launch_bounds__(kStatsThreads) void bn_block_stats_kernel(const T* __restrict__ x, int64_t num_tokens, int hidden,
+                                                                      int rows_per_block, float* __restrict__ partial) {
+    constexpr int V = Elem<T>::kVec;
+    __shared__ float red[3][2][8 * V];
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    const int sub = lane >> 3;                                   // which of the 8 rows of a load
+    const int col = ((int)blockIdx.y * 8 + (lane & 7)) * V;
+    const bool col_ok = col < hidden;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < num_tokens ? r0 + rows_per_block : num_tokens;
+    float pivot[V], s1[V], s2[V];
+    {
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        if (col_ok) raw = *reinterpret_cast<const u32x4_t*>(x + r0 * hidden + col);
+        unpack16<T>(raw, pivot);
+    }
+#pragma unroll
+    for (int v = 0; v < V; ++v) s1[v] = s2[v] = 0.0f;
+    if (col_ok) {
+        constexpr int kBatch = 8;                                // loads issued together: one memory round trip per batch
+        for (int64_t rb = r0 + wave * 8 + sub; rb < r1; rb += 32 * kBatch) {
+            u32x4_t raw[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int64_t r = rb + 32 * i;
+                raw[i] = *reinterpret_cast<const u32x4_t*>(x + (r < r1 ? r : r1 - 1) * hidden + col);
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                if (rb + 32 * i < r1) {
+                    float xv[V];
+                    unpack16<T>(raw[i], xv);
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        const float d = xv[v] - pivot[v];
+                        s1[v] += d;
+                        s2[v] = __builtin_fmaf(d, d, s2[v]);
+                    }
+                }
+            }
+        }
+    }
+    // the 8 row lanes of a wave (lane distance 8, 16, 32), then waves 1..3 -> wave 0 through LDS; fixed order
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+#pragma unroll
+        for (int m = 8; m < kWave; m <<= 1) {
+            s1[v] += __shfl_xor(s1[v], m, kWave);
+            s2[v] += __shfl_xor(s2[v], m, kWave);
+        }
+    }
+    if (wave > 0 && lane < 8) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            red[wave - 1][0][lane * V + v] = s1[v];
+            red[wave - 1][1][lane * V + v] = s2[v];
+        }
+    }
+    __syncthreads();
+    if (wave == 0 && lane < 8 && col_ok) {
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                s1[v] += red[w][0][lane * V + v];
+                s2[v] += red[w][1][lane * V + v];
+            }
+        const float n = (float)(r1 - r0);
+        float* out = partial + (int64_t)blockIdx.x * 2 * hidden;
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            const float m = s1[v] / n;
+            out[col + v] = pivot[v] + m;
+            out[hidden + col + v] = fmaxf(s2[v] - s1[v] * m, 0.0f);
+        }
+    }
+}
+
+// Running statistics live in any of the three dtypes; the gate kernel is not instantiated per statistics dtype.
+__device__ inline float load_stat_rt(const void* p, int i, int dtype) {
+    switch (dtype) {
+        case FMOE_F32: return ((const float*)p)[i];
+        case FMOE_BF16: return Elem<bf16_t>::to_f32(((const bf16_t*)p)[i]);
+        default: return Elem<f16_t>::to_f32(((const f16_t*)p)[i]);
+    }
+}
+__device__ inline void store_stat_rt(void* p, int i, float v, int dtype) {
+    switch (dtype) {
+        case FMOE_F32: ((float*)p)[i] = v; break;
+        case FMOE_BF16: ((bf16_t*)p)[i] = Elem<bf16_t>::from_f32(v); break;
+        default: ((f16_t*)p)[i] = Elem<f16_t>::from_f32(v); break;
+    }
+}
+
+// What the gate kernel's prologue needs to turn block statistics (or running statistics) into mean and 1/std.
+struct GateStats {
+    const float* partial;          // [row_blocks][2][H] from bn_block_stats_kernel (training)
+    int row_blocks, rows_per_block;
+    int64_t num_tokens;
+    int training, stats_dtype;
+    int ready;                     // mean_rstd already holds the statistics (a finalize launch ran): just stage them
+    float momentum, eps;
+    void* running_mean;
+    void* running_var;
+    int64_t* num_batches_tracked;
+    float* mean_rstd;              // [2][H]: kept for a backward pass
+};
+
 template <typename TS> __device__ inline float load_stat(const void* p, int i) { return Elem<TS>::to_f32(((const TS*)p)[i]); }
 template <typename TS> __device__ inline void store_stat(void* p, int i, float v) { ((TS*)p)[i] = Elem<TS>::from_f32(v); }
 
@@ -249,10 +368,9 @@ constexpr int kGateMaxK = 8192;     // mean / rstd of all k are staged in LDS on
 // split != 0: half h of the outputs (columns [h*N/2, (h+1)*N/2)) scores only half h of the normalised activations,
 // w is [N, K/2]: the product-key form in which each sub-key table sees its own half of the query (a block-diagonal gate).
 template <typename T>
-__global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w,
-                                                          const float* __restrict__ mean_rstd, float* __restrict__ logits32,
-                                                          T* __restrict__ logits, int M, int N, int K_full, int tiles_m,
-                                                          int tiles_n, int split, int xcds) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w, GateStats st,
+                                                          float* __restrict__ logits32, T* __restrict__ logits, int M, int N,
+                                                          int K_full, int tiles_m, int tiles_n, int split, int xcds) {
     using Frag = typename Mfma32<T>::Frag;
     constexpr int BM = 64, BN = 64, CH = 2;   // CH = 16-byte packets per thread per tile and operand
     constexpr int D = kGatePrefetch;
@@ -272,10 +390,6 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ 
     const int k_off = (split && n0 >= N / 2) ? K : 0;
     const int k_tiles = (K + kTileK - 1) / kTileK;
     const int kpad = k_tiles * kTileK;
-    for (int i = tid; i < kpad; i += 256) {
-        stats[i] = i < K ? mean_rstd[k_off + i] : 0.0f;
-        stats[kpad + i] = i < K ? mean_rstd[K_full + k_off + i] : 0.0f;
-    }
     u32x4_t ra[D][CH], rb[D][CH];
 
     auto load_global = [&](int kt, int slot) {
@@ -307,6 +421,85 @@ __global__ __launch_bounds__(256) void router_gate_kernel(const T* __restrict__ 
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
     const int frow = lane & 31, fhalf = lane >> 5;
+    // mean and 1/std of this tile's k range into LDS.  One column of tiles per k range also stores them (for a backward
+    // pass) and updates the running statistics: tile row (i / 64) mod tiles_m takes column i, so every column is written
+    // by exactly one workgroup.  Two columns per thread and round: all their block statistics are loaded together (one
+    // memory round trip per round), before the operand prefetch below claims its registers.
+    {
+        constexpr int CPT = 2;
+        const bool keeper = tn == (k_off ? tiles_n / 2 : 0);
+        if (blockIdx.x == 0 && tid == 0 && st.training && !st.ready && st.num_batches_tracked != nullptr) *st.num_batches_tracked += 1;
+        const float n = (float)st.num_tokens;
+        const float full = (float)st.rows_per_block;
+        const float last = (float)(st.num_tokens - (int64_t)(st.row_blocks - 1) * st.rows_per_block);
+        for (int i0 = tid; st.ready && i0 < kpad; i0 += 256) {
+            stats[i0] = i0 < K ? st.mean_rstd[k_off + i0] : 0.0f;
+            stats[kpad + i0] = i0 < K ? st.mean_rstd[K_full + k_off + i0] : 0.0f;
+        }
+        for (int i0 = tid; !st.ready && i0 < kpad; i0 += 256 * CPT) {
+            float mean[CPT], var[CPT], m2[CPT];
+            if (st.training) {
+                float mb[CPT][kFoldMaxRowBlocks], m2b[CPT][kFoldMaxRowBlocks];
+#pragma unroll
+                for (int u = 0; u < CPT; ++u) {
+                    const int i = i0 + u * 256;
+                    const float* pc = st.partial + k_off + (i < K ? i : 0);
+#pragma unroll
+                    for (int b = 0; b < kFoldMaxRowBlocks; ++b) {
+                        const bool ok = b < st.row_blocks;
+                        mb[u][b] = ok ? pc[(int64_t)b * 2 * K_full] : 0.0f;
+                        m2b[u][b] = ok ? pc[(int64_t)b * 2 * K_full + K_full] : 0.0f;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < CPT; ++u) {
+                    float snm = 0.0f;
+#pragma unroll
+                    for (int b = 0; b < kFoldMaxRowBlocks; ++b) {
+                        const float nb = b + 1 < st.row_blocks ? full : (b + 1 == st.row_blocks ? last : 0.0f);
+                        snm = __builtin_fmaf(nb, mb[u][b], snm);
+                    }
+                    mean[u] = snm / n;
+                    float acc2 = 0.0f;
+#pragma unroll
+                    for (int b = 0; b < kFoldMaxRowBlocks; ++b) {
+                        const float nb = b + 1 < st.row_blocks ? full : (b + 1 == st.row_blocks ? last : 0.0f);
+                        const float d = mb[u][b] - mean[u];
+                        acc2 += __builtin_fmaf(nb * d, d, m2b[u][b]);
+                    }
+                    m2[u] = acc2;
+                    var[u] = acc2 / n;                              // biased: what normalises the batch
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < CPT; ++u) {
+                    const int i = i0 + u * 256;
+                    const int c = k_off + (i < K ? i : 0);
+                    mean[u] = load_stat_rt(st.running_mean, c, st.stats_dtype);
+                    var[u] = load_stat_rt(st.running_var, c, st.stats_dtype);
+                    m2[u] = 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < CPT; ++u) {
+                const int i = i0 + u * 256;
+                if (i >= kpad) continue;
+                const int c = k_off + i;
+                const float rstd = 1.0f / sqrtf(var[u] + st.eps);
+                if (i < K && keeper && tm == (i / 64) % tiles_m) {
+                    if (st.training && st.running_mean != nullptr && st.running_var != nullptr) {
+                        const float unbiased = n > 1.0f ? m2[u] / (n - 1.0f) : var[u];
+                        store_stat_rt(st.running_mean, c, (1.0f - st.momentum) * load_stat_rt(st.running_mean, c, st.stats_dtype) + st.momentum * mean[u], st.stats_dtype);
+                        store_stat_rt(st.running_var, c, (1.0f - st.momentum) * load_stat_rt(st.running_var, c, st.stats_dtype) + st.momentum * unbiased, st.stats_dtype);
+                    }
+                    st.mean_rstd[c] = mean[u];
+                    st.mean_rstd[K_full + c] = rstd;
+                }
+                stats[i] = i < K ? mean[u] : 0.0f;
+                stats[kpad + i] = i < K ? rstd : 0.0f;
+            }
+        }
+    }
 #pragma unroll
     for (int d = 0; d < D; ++d) load_global(d, d);
     __syncthreads();               // stats[] visible
@@ -406,6 +599,25 @@ ProloguePlan plan_prologue(int64_t T_, int H, int nk) {
     (void)nk;
     p.bytes = round_up(p.off_mean_rstd + 2 * (size_t)H * 4, 256);
     return p;
+}
+
+// Row blocks of the statistics the gate kernel combines itself: at most kFoldMaxRowBlocks, at least 128 rows each.
+struct BlockStatsPlan { int row_blocks, rows_per_block; };
+BlockStatsPlan plan_block_stats(int64_t T_) {
+    BlockStatsPlan p;
+    int64_t rb = (T_ + 127) / 128;
+    rb = rb < 1 ? 1 : (rb > kFoldMaxRowBlocks ? kFoldMaxRowBlocks : rb);
+    p.rows_per_block = (int)((T_ + rb - 1) / rb);
+    p.row_blocks = (int)((T_ + p.rows_per_block - 1) / p.rows_per_block);
+    return p;
+}
+
+template <typename T>
+void launch_block_stats(const void* x, int64_t T_, int H, const BlockStatsPlan& p, float* partial, hipStream_t stream) {
+    constexpr int V = Elem<T>::kVec;
+    const int strips = (H + 8 * V - 1) / (8 * V);
+    hipLaunchKernelGGL((bn_block_stats_kernel<T>), dim3((unsigned)p.row_blocks, (unsigned)strips), dim3(kStatsThreads), 0, stream,
+                       (const T*)x, T_, H, p.rows_per_block, partial);
 }
 
 template <typename T>
@@ -799,36 +1011,67 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
     float* mean_rstd = (float*)(ws + p.off_mean_rstd);
     float* logits32 = logits_fp32;
 
-    if (training) {
-        switch (dtype) {
-            case FMOE_F32: launch_stats<float>(x, num_tokens, hidden, p, partial, s); break;
-            case FMOE_BF16: launch_stats<bf16_t>(x, num_tokens, hidden, p, partial, s); break;
-            default: launch_stats<f16_t>(x, num_tokens, hidden, p, partial, s); break;
-        }
-        FMOE_CHECK_LAUNCH("fmoe_router_forward(batch statistics)");
-    }
-    switch (stats_dtype) {
-        case FMOE_F32: launch_finalize<float>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
-        case FMOE_BF16: launch_finalize<bf16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
-        default: launch_finalize<f16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
-    }
-    FMOE_CHECK_LAUNCH("fmoe_router_forward(finalize)");
-
     const int M = (int)num_tokens, N = 2 * num_keys;
     if (dtype == FMOE_F32) {
+        if (training) {
+            launch_stats<float>(x, num_tokens, hidden, p, partial, s);
+            FMOE_CHECK_LAUNCH("fmoe_router_forward(batch statistics)");
+        }
+        switch (stats_dtype) {
+            case FMOE_F32: launch_finalize<float>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+            case FMOE_BF16: launch_finalize<bf16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+            default: launch_finalize<f16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+        }
+        FMOE_CHECK_LAUNCH("fmoe_router_forward(finalize)");
         hipLaunchKernelGGL(router_gate_f32_kernel, dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, s, (const float*)x,
                            (const float*)gate_w, (const float*)mean_rstd, logits32, (float*)router_logits, M, N, hidden, split_query);
     } else {
+        const BlockStatsPlan bp = plan_block_stats(num_tokens);
         const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
+        // Every gate workgroup combining the block statistics itself saves a launch, but repeats the combination per
+        // tile: with more than a couple of tiles per CU one finalize launch is cheaper.
+        const bool fold = (int64_t)tiles_m * tiles_n <= 2 * (int64_t)chip_info().cus;
+        if (fold && training) {
+            if (dtype == FMOE_BF16) launch_block_stats<bf16_t>(x, num_tokens, hidden, bp, partial, s);
+            else launch_block_stats<f16_t>(x, num_tokens, hidden, bp, partial, s);
+            FMOE_CHECK_LAUNCH("fmoe_router_forward(batch statistics)");
+        }
+        if (!fold) {
+            if (training) {
+                if (dtype == FMOE_BF16) launch_stats<bf16_t>(x, num_tokens, hidden, p, partial, s);
+                else launch_stats<f16_t>(x, num_tokens, hidden, p, partial, s);
+                FMOE_CHECK_LAUNCH("fmoe_router_forward(batch statistics)");
+            }
+            switch (stats_dtype) {
+                case FMOE_F32: launch_finalize<float>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+                case FMOE_BF16: launch_finalize<bf16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+                default: launch_finalize<f16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
+            }
+            FMOE_CHECK_LAUNCH("fmoe_router_forward(finalize)");
+        }
+        GateStats st;
+        st.ready = fold ? 0 : 1;
+        st.partial = partial;
+        st.row_blocks = bp.row_blocks;
+        st.rows_per_block = bp.rows_per_block;
+        st.num_tokens = num_tokens;
+        st.training = training;
+        st.stats_dtype = stats_dtype;
+        st.momentum = momentum;
+        st.eps = eps;
+        st.running_mean = running_mean;
+        st.running_var = running_var;
+        st.num_batches_tracked = num_batches_tracked;
+        st.mean_rstd = mean_rstd;
         const size_t stats_bytes = (size_t)((hidden + kTileK - 1) / kTileK) * kTileK * 2 * sizeof(float);
         if (dtype == FMOE_BF16)
             hipLaunchKernelGGL((router_gate_kernel<bf16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
-                               (const bf16_t*)x, (const bf16_t*)gate_w, (const float*)mean_rstd, logits32,
-                               (bf16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query, chip_info().xcds);
+                               (const bf16_t*)x, (const bf16_t*)gate_w, st, logits32, (bf16_t*)router_logits, M, N, hidden,
+                               tiles_m, tiles_n, split_query, chip_info().xcds);
         else
             hipLaunchKernelGGL((router_gate_kernel<f16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
-                               (const f16_t*)x, (const f16_t*)gate_w, (const float*)mean_rstd, logits32,
-                               (f16_t*)router_logits, M, N, hidden, tiles_m, tiles_n, split_query, chip_info().xcds);
+                               (const f16_t*)x, (const f16_t*)gate_w, st, logits32, (f16_t*)router_logits, M, N, hidden,
+                               tiles_m, tiles_n, split_query, chip_info().xcds);
     }
     FMOE_CHECK_LAUNCH("fmoe_router_forward(gate)");
     if (top_k == 0) return FMOE_OK;

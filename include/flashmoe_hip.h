@@ -62,7 +62,9 @@ const char* fmoe_last_error(void);
  *   indices    [num_tokens, top_k]        int64      i*num_keys + j; ties to the lower index (tl.argmax rule)
  *   gates      [num_tokens, top_k]        dtype      optional (NULL to skip): exp(score), divided by the
  *                                                    per-token sum when norm_topk_prob != 0
- * Requires 0 <= top_k <= num_keys (same rule as the reference's assert), num_keys <= 65535, top_k <= 256.
+ * Requires 0 <= top_k <= num_keys (same rule as the reference's assert).
+ * Limits of this build (FMOE_ERR_UNSUPPORTED beyond): num_keys <= 65535 and top_k <= 256 (the reference accepts any
+ * top_k <= num_keys, flash_router.py:261-263).
  */
 int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
                      void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream);
@@ -86,6 +88,8 @@ int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, in
  * The normalised activations are rounded to dtype as a stand-alone batch-norm emits them; the product with gate_w,
  * the log-softmax and the pair sums are fp32.  With T == 1 in training mode the call is rejected like
  * nn.BatchNorm1d rejects it.  workspace: fmoe_router_workspace_bytes() bytes, 256-byte aligned.
+ * Limits of this build: num_keys <= 32767, top_k <= 256, num_tokens < 2^31 (FMOE_ERR_UNSUPPORTED beyond); hidden a whole
+ * number of 16-byte packets (FMOE_ERR_ALIGNMENT) and, for the 16-bit dtypes, hidden <= 8192.
  */
 size_t fmoe_router_workspace_bytes(int64_t num_tokens, int hidden, int num_keys);
 
@@ -135,6 +139,13 @@ int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running
  * fmoe_expert_workspace_bytes() gives the scratch fmoe_expert_forward needs for these extents (0 when it takes the
  * row schedule); pass a 256-byte aligned buffer of at least that size.  fmoe_expert_workspace_bytes_algo() gives it
  * for a schedule forced through fmoe_expert_forward_algo().
+ * Limits of this build: hidden a whole number of 16-byte packets (FMOE_ERR_ALIGNMENT); E < 2^31 and T*K < 2^40; and per
+ * schedule (FMOE_ERR_UNSUPPORTED when a call can take none of them, or when the forced one does not apply):
+ *   rows     hidden <= 4096 elements for the 16-bit dtypes, 2048 for fp32
+ *   slices   each table below 4 GiB (rows are addressed with 32-bit byte offsets)
+ *   buckets  rows a multiple of 128 bytes; x and each table below 4 GiB; T*K < 2^31 - 4096; T < 2^24
+ * fmoe_expert_forward picks slices when E*128 bytes fit twice the L2 of one XCD and there are at least 65536 pairs,
+ * else buckets when there are at least 65536 pairs and its limits hold, else rows.
  */
 size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
 size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, int algo);
@@ -221,7 +232,8 @@ int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int h
  *   running_mean / running_var / num_batches_tracked, stats_dtype, training, momentum, eps: as in fmoe_router_forward
  *   out [T,H] dtype; router_logits [T,2*nk] dtype
  *   indices_out [T,K] int64 and gates_out [T,K] dtype: optional (NULL keeps them in the workspace)
- * Requires nk*nk <= E and 0 <= top_k <= nk.
+ * Requires nk*nk <= E and 0 <= top_k <= nk.  The limits of the three stages apply (top_k <= 256, nk <= 32767, the expert
+ * schedules' limits above; hidden and intermediate multiples of 8 for the 16-bit dtypes), and T, E < 2^31.
  */
 size_t fmoe_block_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int num_keys, int64_t num_experts,
                                   int top_k, int dtype);
@@ -259,7 +271,8 @@ int fmoe_pkm_forward(const void* values, const void* routing_weights, const int6
 /* FlashRouterFunc.backward / _flash_router_backward / _bwd_kernel (flash_moe/ops/triton/flash_router.py:317-344,
  * 205-249): drouter_logits [2, T, nk] (dtype), fully written:
  *   [0,t,i] = sum of dscores[t,k] over k with indices[t,k] / nk == i;  [1,t,j] likewise with indices[t,k] % nk.
- * dscores [T, K] dtype, indices [T, K] int64 (ids outside [0, nk*nk) contribute nothing).  num_keys <= 8192. */
+ * dscores [T, K] dtype, indices [T, K] int64 (ids outside [0, nk*nk) contribute nothing).
+ * Limit of this build: num_keys <= 8192 (the forward routes up to 32767). */
 int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64_t num_tokens, int num_keys, int top_k,
                               int dtype, void* drouter_logits, void* stream);
 
@@ -270,7 +283,7 @@ int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64
  *   [0, nk*nk) contribute nothing); logits_fp32 [T, 2*nk]: the fp32 gate logits the forward routed from
  *   (router_logits_fp32 of fmoe_router_forward); dlogits_extra [T, 2*nk] dtype or NULL: gradient of the returned
  *   router logits, added to the result; dlogits_fp32 [T, 2*nk] fp32, fully written: what
- *   fmoe_router_prologue_backward takes.  num_keys <= 8192. */
+ *   fmoe_router_prologue_backward takes.  Limit of this build: num_keys <= 8192. */
 int fmoe_route_backward(const void* dgates, const int64_t* indices, const float* logits_fp32, const void* dlogits_extra,
                         int64_t num_tokens, int num_keys, int top_k, int dtype, int norm_topk_prob, float* dlogits_fp32,
                         void* stream);
@@ -280,7 +293,8 @@ int fmoe_route_backward(const void* dgates, const int64_t* indices, const float*
  * fp32, at byte offset fmoe_router_workspace_stats_offset() of its workspace; pass that as mean_rstd.
  *   dlogits_fp32 [T, 2*nk] fp32 (rounded to dtype for the two GEMMs); dx [T,H], dgate_w [2*nk,H]: dtype.
  * training != 0: batch statistics were used (the gradient flows through mean and variance); else running statistics
- * (constants).  The two GEMMs are rocBLAS calls. */
+ * (constants).  The two GEMMs are rocBLAS calls.
+ * Limits of this build: num_tokens < 2^24; hidden a whole number of 16-byte packets; any num_keys the forward accepts. */
 size_t fmoe_router_workspace_stats_offset(int64_t num_tokens, int hidden, int num_keys);
 size_t fmoe_router_prologue_backward_workspace_bytes(int64_t num_tokens, int hidden, int num_keys, int dtype);
 int fmoe_router_prologue_backward(const float* dlogits_fp32, const void* x, const void* gate_w, const float* mean_rstd,
@@ -305,7 +319,9 @@ int fmoe_mlp_backward(const void* dy, const void* x, const void* gate_w, const v
 
 /* FlashExpertFunc.backward / _flash_expert_backward (flash_moe/ops/triton/flash_expert.py:654-745, kernels :234-525):
  * from dout [T,H] the gradients dx [T,H], ddown, dup [E,H] (rows of experts no pair selects are zero) and
- * dgates [T,K]; indices get none.  Scores are recomputed, not saved.  Requires T*K < 2^31. */
+ * dgates [T,K]; indices get none.  Scores are recomputed, not saved.
+ * Limits of this build: T*K < 2^31, E < 2^31 - 1, hidden a whole number of 16-byte packets and at most 4096 elements for
+ * the 16-bit dtypes, 2048 for fp32 (the per-expert kernel keeps a row in the registers of one wavefront). */
 size_t fmoe_expert_backward_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
 
 int fmoe_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,
