@@ -319,7 +319,8 @@ __global__ __launch_bounds__(256) void expert_backward_gate_kernel(
     if (valid) atomicAdd(&counts[indices[p]], 1);   // integer histogram: the result does not depend on order
 }
 
-// One wave per expert: its rows of ddown and dup, summed over its pairs in ascending pair index.
+// One wave per expert and column chunk (blockIdx.y; NCH * 64 packets each): its rows of ddown and dup, summed over its
+// pairs in ascending pair index.
 template <typename T, int NCH>
 __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kernel(
     const T* __restrict__ dout, const T* __restrict__ x, const float* __restrict__ coef_up,
@@ -331,10 +332,11 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
     const int64_t e = (int64_t)blockIdx.x * kBwdWaves + (threadIdx.x >> 6);
     if (e >= num_experts) return;
     const int packets = hidden / V;
+    const int first = (int)blockIdx.y * NCH * kWave;          // first packet of this column chunk
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
     bool live[NCH];
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) live[c] = c * kWave + lane < packets;
+    for (int c = 0; c < NCH; ++c) live[c] = first + c * kWave + lane < packets;
     float acc_d[NCH][V], acc_u[NCH][V];
 #pragma unroll
     for (int c = 0; c < NCH; ++c)
@@ -366,7 +368,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
                 sd[u] = on ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cd), j)) : 0.0f;
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
-                    const int p = c * kWave + lane;
+                    const int p = first + c * kWave + lane;
                     xq[u][c] = (on && live[c]) ? reinterpret_cast<const u32x4_t*>(x + t * hidden)[p] : zero4;
                     gq[u][c] = (on && live[c]) ? reinterpret_cast<const u32x4_t*>(dout + t * hidden)[p] : zero4;
                 }
@@ -382,7 +384,7 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void expert_backward_weight_kerne
     }
 #pragma unroll
     for (int c = 0; c < NCH; ++c) {
-        const int p = c * kWave + lane;
+        const int p = first + c * kWave + lane;
         if (live[c]) {
             reinterpret_cast<u32x4_t*>(ddown + e * hidden)[p] = pack16<T>(acc_d[c]);
             reinterpret_cast<u32x4_t*>(dup + e * hidden)[p] = pack16<T>(acc_u[c]);
@@ -436,7 +438,7 @@ int launch_expert_backward(const void* dout, const void* x, const void* down, co
     const int nch = (H / V + kWave - 1) / kWave;
     const dim3 block(kBwdWaves * kWave);
     const dim3 token_grid((unsigned)((T_ + kBwdWaves - 1) / kBwdWaves));
-    const dim3 expert_grid((unsigned)((E + kBwdWaves - 1) / kBwdWaves));
+    const dim3 expert_grid((unsigned)((E + kBwdWaves - 1) / kBwdWaves), (unsigned)((nch + 7) / 8));   // y: column chunks of long rows
 
     if (int rc = bucket_clear(bucket_ws, E, stream)) return rc;
     if (p.slices) {
@@ -586,8 +588,10 @@ extern "C" int fmoe_expert_backward(const void* dout, const void* x, const void*
                  "fmoe_expert_backward: bad shape T=%lld H=%d E=%lld K=%d", (long long)num_tokens, hidden, (long long)num_experts, top_k);
     const int vec = (int)(16 / dtype_size(dtype));
     FMOE_REQUIRE(hidden % vec == 0, FMOE_ERR_ALIGNMENT, "fmoe_expert_backward: hidden=%d must be a multiple of %d (16-byte rows)", hidden, vec);
-    FMOE_REQUIRE(hidden <= 8 * kWave * vec, FMOE_ERR_UNSUPPORTED, "fmoe_expert_backward: hidden=%d exceeds the %d elements per row this build supports",
-                 hidden, 8 * kWave * vec);
+    // rows too long for the per-token row kernel take the column-slice kernels, which need 32-bit row offsets
+    FMOE_REQUIRE(hidden <= 8 * kWave * vec || num_tokens == 0 || top_k == 0 || expert_slices_usable(num_tokens, hidden, num_experts, top_k, dtype),
+                 FMOE_ERR_UNSUPPORTED, "fmoe_expert_backward: rows of more than %d elements need tables below 4 GiB (hidden=%d, E=%lld)",
+                 8 * kWave * vec, hidden, (long long)num_experts);
     FMOE_REQUIRE(num_experts < (1ll << 31) - 1 && (int64_t)num_tokens * top_k < (1ll << 31), FMOE_ERR_UNSUPPORTED,
                  "fmoe_expert_backward: E=%lld or T*K=%lld >= 2^31", (long long)num_experts, (long long)num_tokens * top_k);
     FMOE_REQUIRE(ddown && dup && down && up && (num_tokens == 0 || (dx && x && dout)), FMOE_ERR_NULL_POINTER,

@@ -1022,13 +1022,20 @@ bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= 2 * chip_info(
 // rows are addressed with 32-bit byte offsets below kBadOffset
 bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
 
+// the row kernels keep a whole row in the registers of one wavefront: at most 8 packets of 16 bytes per lane
+bool rows_possible(int H, size_t elt) { return (size_t)H * elt <= (size_t)8 * kWave * 16; }
+// column slices: when they pay, and for rows too long for the row kernels whatever the problem size
+bool slices_chosen(int64_t T_, int H, int64_t E, int K, size_t elt) {
+    return slices_possible(E, H, elt) && (slices_pay(T_, E, K) || !rows_possible(H, elt));
+}
+
 // Which schedule a call takes.  A forced schedule that cannot run these extents is reported by the dispatcher; AUTO
 // falls back to whole rows.
 bool buckets_pay(int64_t T_, int64_t E, int K) { return !slices_pay(T_, E, K) && T_ * K >= (1ll << 16); }
 int choose_schedule(int algo, int64_t T_, int H, int64_t E, int K, size_t elt) {
     if (K == 0) return FMOE_EXPERT_ROWS;
     if (algo != FMOE_EXPERT_AUTO) return algo;
-    if (slices_pay(T_, E, K) && slices_possible(E, H, elt)) return FMOE_EXPERT_SLICES;
+    if (slices_chosen(T_, H, E, K, elt)) return FMOE_EXPERT_SLICES;
     if (buckets_pay(T_, E, K) && bucketed_possible(T_, E, H, K, elt)) return FMOE_EXPERT_BUCKETS;
     return FMOE_EXPERT_ROWS;
 }
@@ -1036,7 +1043,7 @@ int choose_schedule(int algo, int64_t T_, int H, int64_t E, int K, size_t elt) {
 }  // namespace
 
 bool expert_slices_usable(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
-    return top_k > 0 && slices_pay(num_tokens, num_experts, top_k) && slices_possible(num_experts, hidden, dtype_size(dtype));
+    return top_k > 0 && slices_chosen(num_tokens, hidden, num_experts, top_k, dtype_size(dtype));
 }
 
 uint32_t* expert_workspace_offsets(void* workspace) { return (uint32_t*)workspace; }   // SlicePlan::off_idx32 == 0

@@ -141,11 +141,12 @@ int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running
  * for a schedule forced through fmoe_expert_forward_algo().
  * Limits of this build: hidden a whole number of 16-byte packets (FMOE_ERR_ALIGNMENT); E < 2^31 and T*K < 2^40; and per
  * schedule (FMOE_ERR_UNSUPPORTED when a call can take none of them, or when the forced one does not apply):
- *   rows     hidden <= 4096 elements for the 16-bit dtypes, 2048 for fp32
+ *   rows     rows of at most 8192 bytes (hidden <= 4096 for the 16-bit dtypes, 2048 for fp32)
  *   slices   each table below 4 GiB (rows are addressed with 32-bit byte offsets)
  *   buckets  rows a multiple of 128 bytes; x and each table below 4 GiB; T*K < 2^31 - 4096; T < 2^24
- * fmoe_expert_forward picks slices when E*128 bytes fit twice the L2 of one XCD and there are at least 65536 pairs,
- * else buckets when there are at least 65536 pairs and its limits hold, else rows.
+ * fmoe_expert_forward picks slices when E*128 bytes fit twice the L2 of one XCD and there are at least 65536 pairs, or
+ * when the rows are too long for the row schedule; else buckets when there are at least 65536 pairs and its limits
+ * hold; else rows.  So any hidden size works as long as each table stays below 4 GiB.
  */
 size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
 size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, int algo);
@@ -320,8 +321,8 @@ int fmoe_mlp_backward(const void* dy, const void* x, const void* gate_w, const v
 /* FlashExpertFunc.backward / _flash_expert_backward (flash_moe/ops/triton/flash_expert.py:654-745, kernels :234-525):
  * from dout [T,H] the gradients dx [T,H], ddown, dup [E,H] (rows of experts no pair selects are zero) and
  * dgates [T,K]; indices get none.  Scores are recomputed, not saved.
- * Limits of this build: T*K < 2^31, E < 2^31 - 1, hidden a whole number of 16-byte packets and at most 4096 elements for
- * the 16-bit dtypes, 2048 for fp32 (the per-expert kernel keeps a row in the registers of one wavefront). */
+ * Limits of this build: T*K < 2^31, E < 2^31 - 1, hidden a whole number of 16-byte packets; rows of more than 8192 bytes
+ * (hidden > 4096 for the 16-bit dtypes, 2048 for fp32) need tables below 4 GiB. */
 size_t fmoe_expert_backward_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
 
 int fmoe_expert_backward(const void* dout, const void* x, const void* down, const void* up, const int64_t* indices,

@@ -143,7 +143,8 @@ def expert_case(T, H, E, K, dtype, seed, duplicates=False):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,E,K,dup", [(64, 128, 256, 8, False), (200, 256, 64, 16, True), (33, 1024, 4096, 5, False),
-                                         (16, 2048, 512, 4, False)])
+                                         (16, 2048, 512, 4, False),
+                                         (12, 8192, 48, 4, False), (20, 5120, 40, 3, True)])   # rows beyond one wave's registers
 def test_expert_backward(dtype, T, H, E, K, dup):
     from flash_moe.ops import flash_expert_func
     from flash_moe.ops.hip.flash_expert import expert_backward

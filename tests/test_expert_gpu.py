@@ -51,6 +51,21 @@ def test_expert_matches_oracle(dtype, T, H, E, K, algo):
     assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 5e-4}[dtype], fro
 
 
+@pytest.mark.parametrize("dtype,H", [(torch.bfloat16, 8192), (torch.bfloat16, 5120), (torch.float16, 4104), (torch.float32, 2304)])
+def test_expert_long_rows_take_the_column_slices(dtype, H):
+    # rows of more than 8192 bytes do not fit the registers of the one-wave-per-token kernel: the op takes the column-slice
+    # kernels for them whatever the problem size (the reference has no limit on hidden_size); forcing rows is refused
+    T, E, K = 24, 96, 6
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=H)
+    x, wd, wu, g = (t.to(dtype) for t in (x, wd, wu, g))
+    got = run(x, wd, wu, idx, g, "auto")
+    assert_output_close(got, orc.expert_forward(x, wd, wu, idx, g), dtype, "expert, long rows")
+    fro = rel_fro(got, truth64(x, wd, wu, idx, g))
+    assert fro < {torch.float32: 2e-6, torch.bfloat16: 4e-3, torch.float16: 5e-4}[dtype], fro
+    with pytest.raises(ValueError, match="elements per row"):
+        run(x, wd, wu, idx, g, "rows")
+
+
 @pytest.mark.parametrize("algo", SCHEDULES)
 def test_expert_reference_test_distribution(algo):
     # distributions of the reference's expert benchmark (tests/test_expert.py:160-175): x ~ N(0,0.5),

@@ -55,6 +55,8 @@ def check_fp32_case(lp, nk, K):
     (8192, 128, 64),                           # C2
     (300, 512, 128),                           # C5 keys, few tokens
     (77, 100, 37), (5, 13, 13), (64, 8, 1), (33, 256, 200), (1, 128, 64), (1030, 64, 64),
+    # every top-k kernel variant: lists in registers (nk <= 128 or <= 512, K <= 64 or <= 128) and the group scan beyond
+    (200, 128, 128), (150, 512, 64), (40, 300, 100), (64, 600, 64), (48, 520, 128),
 ])
 def test_router_fp32_log_probs(T, nk, K):
     check_fp32_case(orc.make_router_inputs(T, nk, seed=T + nk), nk, K)
