@@ -92,7 +92,10 @@ def test_expert_argument_checks():
     assert f(a, a, a, None, a, 4, 64, 16, 2, _C.BF16, a, None, 0, None) == -1
     assert f(a, a, a, a, a, 4, 60, 16, 2, _C.BF16, a, None, 0, None) == -6          # row not 16-byte multiple
     assert f(a + 2, a, a, a, a, 4, 64, 16, 2, _C.BF16, a, None, 0, None) == -6      # misaligned pointer
-    assert f(a, a, a, a, a, 4, 1 << 20, 16, 2, _C.BF16, a, None, 0, None) == -5      # hidden too large
+    # rows too long for the row kernels take the column slices, which need their workspace; forcing rows is refused
+    assert f(a, a, a, a, a, 4, 1 << 20, 16, 2, _C.BF16, a, None, 0, None) == -7
+    assert lib.fmoe_expert_workspace_bytes(4, 1 << 20, 16, 2, _C.BF16) > 0
+    assert lib.fmoe_expert_forward_algo(a, a, a, a, a, 4, 1 << 20, 16, 2, _C.BF16, a, None, 0, _C.EXPERT_ROWS, None) == -5
     assert f(None, None, None, None, None, 0, 64, 16, 2, _C.BF16, None, None, 0, None) == 0
     assert isinstance(lib.fmoe_expert_workspace_bytes(1024, 1024, 16384, 64, _C.BF16), int)
     # the size follows the schedule: column slices when a slice of the table fits L2 and there are enough pairs, else none
