@@ -200,7 +200,8 @@ def test_backward_argument_checks():
     assert ecall(dtype=3) == -4
     assert ecall(H=0) == -2
     assert ecall(H=60) == -6
-    assert ecall(H=8192) == -5
+    assert ecall(H=8192) == -7                     # long rows take the column-slice kernels: a larger workspace
+    assert ecall(H=8192, E=1 << 19) == -5          # ... which cannot address tables of 4 GiB or more
     assert ecall(dout=None) == -1
     assert ecall(ws_bytes=need - 1) == -7
     mneed = lib.fmoe_mlp_backward_workspace_bytes(8, 64, 128, _C.BF16)
