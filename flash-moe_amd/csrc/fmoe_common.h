@@ -48,6 +48,8 @@ const ChipInfo& chip_info();
 int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
                               int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, uint32_t* row_offsets,
                               uint32_t row_bytes, hipStream_t stream);
+// Whether a top-k kernel exists for these extents: top_k <= 256 with any num_keys, or top_k <= 1024 with num_keys <= 8192.
+bool router_topk_supported(int num_keys, int top_k);
 
 // The fused router (fmoe_router_forward) with the optional row-offset output; defined in fmoe_router_prologue.hip.
 int router_forward_impl(const void* x, const void* gate_w, void* running_mean, void* running_var,

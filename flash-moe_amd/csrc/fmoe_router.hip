@@ -446,6 +446,127 @@ __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// top_k beyond 256 (up to 1024, with num_keys up to 8192): one workgroup per token, every ordering is a bitonic sort of
+// the 64-bit keys in LDS.  Same pruning, same keys and therefore the same result as the kernels above; an order of
+// magnitude slower per token, for shapes none of the reference's configurations use.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int kBigThreads = 1024;
+constexpr int kBigMaxKeys = 8192;      // 64 KiB of keys
+constexpr int kBigMaxTopK = 1024;      // sum_{i<=1024} floor(1024/i) = 7689 candidates <= kBigMaxKeys
+
+// descending bitonic sort of keys[0..m), m a power of two, by the whole workgroup
+__device__ inline void block_sort_desc(uint64_t* keys, int m) {
+    for (int k = 2; k <= m; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = (int)threadIdx.x; i < m / 2; i += (int)blockDim.x) {
+                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1)), hi = lo | j;
+                const uint64_t a = keys[lo], b = keys[hi];
+                if ((a < b) == ((lo & k) == 0)) {
+                    keys[lo] = b;
+                    keys[hi] = a;
+                }
+            }
+            __syncthreads();
+        }
+}
+
+template <typename T, typename TG, bool FROM_LOGITS>
+__global__ __launch_bounds__(kBigThreads) void router_topk_big_kernel(
+    const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
+    int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets,
+    uint32_t row_bytes) {
+    __shared__ uint64_t keys[kBigMaxKeys];
+    __shared__ float half_score[2][kBigMaxTopK];
+    __shared__ uint32_t half_index[2][kBigMaxTopK];
+    __shared__ uint32_t row_start[kBigMaxTopK + 1];    // candidates of rank i in half 0 start here; row i has top_k/(i+1)
+    __shared__ float stat[2];
+    const int tid = (int)threadIdx.x, lane = lane_id();
+    for (int i = tid; i <= top_k; i += kBigThreads) {
+        uint32_t off = 0;
+        for (int q = 0; q < i; ++q) off += (uint32_t)(top_k / (q + 1));
+        row_start[i] = off;
+    }
+    int m_half = 64, m_cand = 64;
+    while (m_half < nk) m_half <<= 1;
+    while (m_cand < num_cand) m_cand <<= 1;
+    const int kept = top_k < nk ? top_k : nk;           // ranks of a half the candidates can name
+    __syncthreads();
+
+    for (int64_t token = blockIdx.x; token < num_tokens; token += gridDim.x) {
+        for (int h = 0; h < 2; ++h) {
+            const T* row = FROM_LOGITS ? lp + (token * 2 + h) * nk : lp + ((int64_t)h * num_tokens + token) * nk;
+            if (FROM_LOGITS) {
+                // by one wave, in the order the one-wave-per-token kernels use: identical log-probabilities
+                if (tid < kWave) {
+                    float mx = -INFINITY;
+                    for (int p = lane; p < nk; p += kWave) mx = fmaxf(mx, Elem<T>::to_f32(row[p]));
+                    mx = wave_max(mx);
+                    float se = 0.0f;
+                    for (int p = lane; p < nk; p += kWave) se += expf(Elem<T>::to_f32(row[p]) - mx);
+                    const float lse = logf(wave_sum(se));
+                    if (lane == 0) {
+                        stat[0] = mx;
+                        stat[1] = lse;
+                    }
+                }
+                __syncthreads();
+            }
+            const float shift = FROM_LOGITS ? stat[0] : 0.0f, lse = FROM_LOGITS ? stat[1] : 0.0f;
+            for (int p = tid; p < m_half; p += kBigThreads) {
+                uint64_t key = 0ull;
+                if (p < nk) {
+                    const float v = Elem<T>::to_f32(row[p]);
+                    key = make_key(FROM_LOGITS ? (v - shift) - lse : v, (uint32_t)p);
+                }
+                keys[p] = key;
+            }
+            __syncthreads();
+            block_sort_desc(keys, m_half);
+            for (int r = tid; r < kept; r += kBigThreads) {
+                half_score[h][r] = key_score(keys[r]);
+                half_index[h][r] = key_index(keys[r]);
+            }
+            __syncthreads();
+        }
+        for (int c = tid; c < m_cand; c += kBigThreads) keys[c] = 0ull;
+        __syncthreads();
+        for (int i = tid; i < kept; i += kBigThreads) {
+            const uint32_t at = row_start[i];
+            int n = (int)(row_start[i + 1] - at);
+            n = n < kept ? n : kept;                                    // half 1 has only `kept` ranks
+            const float si = half_score[0][i];
+            const uint32_t base = half_index[0][i] * (uint32_t)nk;
+            for (int j = 0; j < n; ++j)
+                keys[at + j] = make_key(round_through<T>(si + half_score[1][j]), base + half_index[1][j]);
+        }
+        __syncthreads();
+        block_sort_desc(keys, m_cand);
+        if (tid < kWave) {
+            float total = 0.0f;
+            if (gates != nullptr && norm_topk_prob) {
+                for (int p = lane; p < top_k; p += kWave) total += expf(key_score(keys[p]));
+                total = wave_sum(total);
+            }
+            stat[0] = total;
+        }
+        __syncthreads();
+        const float total = stat[0];
+        for (int p = tid; p < top_k; p += kBigThreads) {
+            const uint64_t key = keys[p];
+            const int64_t o = token * top_k + p;
+            scores[o] = Elem<T>::from_f32(key_score(key));
+            indices[o] = (int64_t)key_index(key);
+            if (row_offsets != nullptr) row_offsets[o] = key_index(key) * row_bytes;
+            if (gates != nullptr) {
+                const float e = expf(key_score(key));
+                gates[o] = Elem<TG>::from_f32(norm_topk_prob ? e / total : e);
+            }
+        }
+        __syncthreads();
+    }
+}
+
 int count_candidates(int top_k) {
     int n = 0;
     for (int i = 1; i <= top_k; ++i) n += top_k / i;
@@ -460,6 +581,13 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
     const int64_t max_blocks = (int64_t)chip_info().cus * 8;   // a few resident blocks per CU; the kernel loops over tokens
     const dim3 grid((unsigned)(blocks_needed < max_blocks ? blocks_needed : max_blocks));
     const dim3 block(kRouterWaves * kWave);
+    if (K > kMaxTopK) {      // the workgroup-per-token kernel; its limits are checked by the callers
+        const int64_t big_blocks = T_ < (int64_t)chip_info().cus * 2 ? T_ : (int64_t)chip_info().cus * 2;
+        hipLaunchKernelGGL((router_topk_big_kernel<T, TG, FROM_LOGITS>), dim3((unsigned)big_blocks), dim3(kBigThreads), 0, stream,
+                           (const T*)lp, T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes);
+        FMOE_CHECK_LAUNCH("fmoe_router_topk");
+        return FMOE_OK;
+    }
     // lists that fit the registers of a wave take the threshold selection
 #define FMOE_LAUNCH_SELECT(RK_, RH_, RC_)                                                                              \
     hipLaunchKernelGGL((router_select_kernel<T, TG, RK_, RH_, RC_, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, \
@@ -490,6 +618,10 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
 
 }  // namespace
 
+bool router_topk_supported(int num_keys, int top_k) {
+    return top_k <= kMaxTopK || (top_k <= kBigMaxTopK && num_keys <= kBigMaxKeys);
+}
+
 int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
                               int64_t* indices, void* gates, int gate_dtype, int norm_topk_prob, uint32_t* row_offsets,
                               uint32_t row_bytes, hipStream_t stream) {
@@ -512,7 +644,9 @@ extern "C" int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int n
     FMOE_REQUIRE(top_k >= 0 && top_k <= num_keys, FMOE_ERR_TOPK_RANGE,
                  "num_experts_per_tok should be in [0, %d], but got %d", num_keys, top_k);
     FMOE_REQUIRE(num_keys <= 65535, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk: num_keys=%d > 65535", num_keys);
-    FMOE_REQUIRE(top_k <= kMaxTopK, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk: top_k=%d > %d", top_k, kMaxTopK);
+    FMOE_REQUIRE(router_topk_supported(num_keys, top_k), FMOE_ERR_UNSUPPORTED,
+                 "fmoe_router_topk: top_k=%d > %d needs top_k <= %d and num_keys <= %d (num_keys=%d)", top_k, kMaxTopK, kBigMaxTopK,
+                 kBigMaxKeys, num_keys);
     if (num_tokens == 0 || top_k == 0) return FMOE_OK;
     FMOE_REQUIRE(log_probs && scores && indices, FMOE_ERR_NULL_POINTER, "fmoe_router_topk: null tensor pointer");
     hipStream_t s = (hipStream_t)stream;

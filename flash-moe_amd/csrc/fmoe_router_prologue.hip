@@ -988,7 +988,7 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
                  "num_experts_per_tok should be in [0, %d], but got %d", num_keys, top_k);
     FMOE_REQUIRE(dtype == FMOE_F32 || hidden <= kGateMaxK, FMOE_ERR_UNSUPPORTED,
                  "fmoe_router_forward: hidden=%d > %d for 16-bit activations", hidden, kGateMaxK);
-    FMOE_REQUIRE(num_keys <= 32767 && top_k <= 256 && num_tokens < (1ll << 31), FMOE_ERR_UNSUPPORTED,
+    FMOE_REQUIRE(num_keys <= 32767 && router_topk_supported(num_keys, top_k) && num_tokens < (1ll << 31), FMOE_ERR_UNSUPPORTED,
                  "fmoe_router_forward: nk=%d top_k=%d T=%lld beyond what the kernels are built for", num_keys, top_k,
                  (long long)num_tokens);
     if (num_tokens == 0) return FMOE_OK;

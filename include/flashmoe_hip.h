@@ -63,8 +63,9 @@ const char* fmoe_last_error(void);
  *   gates      [num_tokens, top_k]        dtype      optional (NULL to skip): exp(score), divided by the
  *                                                    per-token sum when norm_topk_prob != 0
  * Requires 0 <= top_k <= num_keys (same rule as the reference's assert).
- * Limits of this build (FMOE_ERR_UNSUPPORTED beyond): num_keys <= 65535 and top_k <= 256 (the reference accepts any
- * top_k <= num_keys, flash_router.py:261-263).
+ * Limits of this build (FMOE_ERR_UNSUPPORTED beyond): num_keys <= 65535; top_k <= 256, or top_k <= 1024 with
+ * num_keys <= 8192 (a slower workgroup-per-token kernel).  The reference accepts any top_k <= num_keys
+ * (flash_router.py:261-263).
  */
 int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
                      void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream);
@@ -88,7 +89,7 @@ int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, in
  * The normalised activations are rounded to dtype as a stand-alone batch-norm emits them; the product with gate_w,
  * the log-softmax and the pair sums are fp32.  With T == 1 in training mode the call is rejected like
  * nn.BatchNorm1d rejects it.  workspace: fmoe_router_workspace_bytes() bytes, 256-byte aligned.
- * Limits of this build: num_keys <= 32767, top_k <= 256, num_tokens < 2^31 (FMOE_ERR_UNSUPPORTED beyond); hidden a whole
+ * Limits of this build: num_keys <= 32767, top_k as in fmoe_router_topk, num_tokens < 2^31 (FMOE_ERR_UNSUPPORTED beyond); hidden a whole
  * number of 16-byte packets (FMOE_ERR_ALIGNMENT) and, for the 16-bit dtypes, hidden <= 8192.
  */
 size_t fmoe_router_workspace_bytes(int64_t num_tokens, int hidden, int num_keys);
@@ -233,7 +234,7 @@ int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int h
  *   running_mean / running_var / num_batches_tracked, stats_dtype, training, momentum, eps: as in fmoe_router_forward
  *   out [T,H] dtype; router_logits [T,2*nk] dtype
  *   indices_out [T,K] int64 and gates_out [T,K] dtype: optional (NULL keeps them in the workspace)
- * Requires nk*nk <= E and 0 <= top_k <= nk.  The limits of the three stages apply (top_k <= 256, nk <= 32767, the expert
+ * Requires nk*nk <= E and 0 <= top_k <= nk.  The limits of the three stages apply (top_k <= 256 or <= 1024 with nk <= 8192, nk <= 32767, the expert
  * schedules' limits above; hidden and intermediate multiples of 8 for the 16-bit dtypes), and T, E < 2^31.
  */
 size_t fmoe_block_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int num_keys, int64_t num_experts,

@@ -134,6 +134,22 @@ def test_block_c5_shape_fewer_tokens():
     stagewise_check(m, w, x, 128, True, dtype)
 
 
+def test_block_with_more_than_256_experts_per_token():
+    # num_experts_per_tok may be anything up to the number of keys in the reference (flash_router.py:261-263); beyond 256
+    # the router takes its workgroup-per-token kernel
+    m, w = build(256, 512, 320 * 320, 300, True, torch.float32)
+    x = torch.randn(1, 48, 256, generator=torch.Generator().manual_seed(0))
+    stagewise_check(m, w, x, 300, True, torch.float32)
+
+
+def test_block_with_long_rows():
+    # hidden_size 5120: rows of 10240 bytes, longer than one wavefront's registers hold; the expert stage takes column slices
+    dtype = torch.bfloat16
+    m, w = build(5120, 1024, 1024, 8, False, dtype)
+    x = torch.randn(1, 40, 5120, generator=torch.Generator().manual_seed(0)).to(dtype)
+    stagewise_check(m, w, x, 8, False, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,H,I,E,K", [(1024, 256, 512, 4096, 64),     # column-slice expert schedule
                                        (96, 128, 256, 1024, 8),        # row-gather expert schedule
