@@ -901,6 +901,9 @@ struct BucketedPlan {
     bool sweep;
 };
 
+// the row kernels keep a whole row in the registers of one wavefront: at most 8 packets of 16 bytes per lane
+bool rows_possible(int H, size_t elt) { return (size_t)H * elt <= (size_t)8 * kWave * 16; }
+
 // The sweep needs 16-bit rows of whole 128-byte bands, at most 256 pairs per token, ids below 2^22 and lists below 4 GiB.
 bool sweep_possible(int64_t T_, int H, int64_t E, int K, size_t elt) {
     const int64_t padded = (T_ + kSweepTokens - 1) / kSweepTokens * kSweepTokens;
@@ -944,7 +947,8 @@ BucketedPlan plan_bucketed(int64_t T_, int H, int64_t E, int K, size_t elt) {
 bool bucketed_possible(int64_t T_, int64_t E, int H, int K, size_t elt) {
     return (H * elt) % 128 == 0 &&      // whole 128-byte bands
            (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset && (uint64_t)T_ * (uint64_t)H * elt < (uint64_t)kBadOffset &&
-           T_ * (int64_t)K < (1ll << 31) - 4096 && E < (1ll << 31) - 1 && T_ <= (int64_t)kEntryTokenMask;
+           T_ * (int64_t)K < (1ll << 31) - 4096 && E < (1ll << 31) - 1 && T_ <= (int64_t)kEntryTokenMask &&
+           (sweep_possible(T_, H, E, K, elt) || rows_possible(H, elt));     // its second phase: the sweep, or the row kernel
 }
 
 template <typename T>
@@ -1022,8 +1026,6 @@ bool slices_pay(int64_t T_, int64_t E, int K) { return E * 128 <= 2 * chip_info(
 // rows are addressed with 32-bit byte offsets below kBadOffset
 bool slices_possible(int64_t E, int H, size_t elt) { return (uint64_t)E * (uint64_t)H * elt < (uint64_t)kBadOffset; }
 
-// the row kernels keep a whole row in the registers of one wavefront: at most 8 packets of 16 bytes per lane
-bool rows_possible(int H, size_t elt) { return (size_t)H * elt <= (size_t)8 * kWave * 16; }
 // column slices: when they pay, and for rows too long for the row kernels whatever the problem size
 bool slices_chosen(int64_t T_, int H, int64_t E, int K, size_t elt) {
     return slices_possible(E, H, elt) && (slices_pay(T_, E, K) || !rows_possible(H, elt));
@@ -1139,7 +1141,7 @@ int expert_dispatch(const char* who, int act, const void* x, const void* down, c
     FMOE_REQUIRE(schedule != FMOE_EXPERT_SLICES || slices_possible(num_experts, hidden, elt), FMOE_ERR_UNSUPPORTED,
                  "%s: tables of 4 GiB or more cannot use the column-slice schedule", who);
     FMOE_REQUIRE(schedule != FMOE_EXPERT_BUCKETS || bucketed_possible(num_tokens, num_experts, hidden, top_k, elt),
-                 FMOE_ERR_UNSUPPORTED, "%s: the bucketed schedule needs rows that are multiples of 128 bytes, x and each table below 4 GiB and fewer than 2^31 pairs", who);
+                 FMOE_ERR_UNSUPPORTED, "%s: the bucketed schedule needs rows that are multiples of 128 bytes (16-bit, or at most 8192 bytes), x and each table below 4 GiB and fewer than 2^31 pairs", who);
     if (schedule == FMOE_EXPERT_BUCKETS) {
         const size_t need = fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, dtype, FMOE_EXPERT_BUCKETS);
         FMOE_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
