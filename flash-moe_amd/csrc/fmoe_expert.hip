@@ -252,13 +252,31 @@ __global__ __launch_bounds__(256) void expert_prepare_kernel(const int64_t* __re
     }
 }
 
-// Workgroup b runs on XCD b % xcds (ids are dealt round-robin): XCD x takes slices x, x + xcds, ...
+// Workgroup b runs on XCD b % xcds (ids are dealt round-robin): XCD x takes slices x, x + xcds, ... for whole rounds of
+// xcds slices.  The slices left over after the last whole round (fewer than xcds) would leave XCDs idle: each of them is
+// shared by xcds / left XCDs instead, which take interleaved token blocks of it.
+__host__ __device__ inline int slice_parts(int num_slices, int xcds) {
+    const int left = num_slices % xcds;
+    return left ? xcds / left : 1;
+}
+__host__ __device__ inline int slice_grid_rows(int num_slices, int blocks_per_slice, int xcds) {   // grid = xcds * rows
+    const int parts = slice_parts(num_slices, xcds);
+    return (num_slices / xcds) * blocks_per_slice + (num_slices % xcds ? (blocks_per_slice + parts - 1) / parts : 0);
+}
 __device__ inline bool slice_of_block(int num_slices, int blocks_per_slice, int xcds, int& slice, int& tb) {
     const int b = (int)blockIdx.x;
-    const int j = b / xcds;
-    slice = b % xcds + xcds * (j / blocks_per_slice);
-    tb = j % blocks_per_slice;
-    return slice < num_slices;
+    const int x = b % xcds, j = b / xcds;
+    const int whole = num_slices / xcds;
+    if (j < whole * blocks_per_slice) {
+        slice = x + xcds * (j / blocks_per_slice);
+        tb = j % blocks_per_slice;
+        return true;
+    }
+    const int left = num_slices % xcds, parts = slice_parts(num_slices, xcds);
+    if (left == 0 || x / left >= parts) return false;
+    slice = whole * xcds + x % left;
+    tb = (j - whole * blocks_per_slice) * parts + x / left;
+    return tb < blocks_per_slice;
 }
 
 // p[u] holds, in each of the CL lanes of a chunk group, that lane's share of pair u's dot product.  Returns in
@@ -443,7 +461,7 @@ SlicePlan plan_slices(int64_t T_, int H, int64_t E, int K, size_t elt) {
     const int64_t want = (T_ + 3) / 4;                       // at least one token per wave
     p.blocks_per_slice = (int)(want < 1024 ? want : 1024);   // 256 blocks of 4 waves fill one XCD; a few rounds of them
     p.tokens_per_block = (int)((T_ + p.blocks_per_slice - 1) / p.blocks_per_slice);
-    p.grid = (unsigned)(p.xcds * p.blocks_per_slice * ((p.num_slices + p.xcds - 1) / p.xcds));
+    p.grid = (unsigned)(p.xcds * slice_grid_rows(p.num_slices, p.blocks_per_slice, p.xcds));
     const size_t pairs = (size_t)T_ * (size_t)K;
     p.off_idx32 = 0;
     p.off_a = round_up(p.off_idx32 + pairs * 4, 256);
