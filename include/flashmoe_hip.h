@@ -146,8 +146,9 @@ int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running
  *   slices   each table below 4 GiB (rows are addressed with 32-bit byte offsets)
  *   buckets  rows a multiple of 128 bytes; x and each table below 4 GiB; T*K < 2^31 - 4096; T < 2^24
  * fmoe_expert_forward picks slices when E*128 bytes fit twice the L2 of one XCD and there are at least 65536 pairs, or
- * when the rows are too long for the row schedule; else buckets when there are at least 65536 pairs and its limits
- * hold; else rows.  So any hidden size works as long as each table stays below 4 GiB.
+ * when the rows are too long for the row schedule; else buckets when there are at least 65536 pairs and 12 pairs per
+ * expert (each table row then serves enough pairs to pay for the grouping) and its limits hold; else rows.  So any
+ * hidden size works as long as each table stays below 4 GiB.
  */
 size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
 size_t fmoe_expert_workspace_bytes_algo(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, int algo);
