@@ -22,7 +22,8 @@ def pkm_reference(values, w, idx):
 CASES = [(64, 128, 256, 8),            # row schedule
          (1024, 256, 4096, 64),        # column-slice schedule (T*K >= 65536, slice fits L2)
          (33, 1024, 1000, 5),          # ragged
-         (16, 2048, 512, 4)]
+         (16, 2048, 512, 4),
+         (20, 5120, 96, 6)]            # rows beyond one wavefront's registers: column slices whatever the size
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
