@@ -169,8 +169,8 @@ def stage_kernels(m, x):
 
 # kernels behind each timed C-ABI call, as they appear in the rocprofv3 summaries under profiles/
 LAUNCHES = {
-    "router_forward": ["bn_partial_kernel", "bn_finalize_kernel", "router_gate_kernel", "router_topk_kernel"],
-    "router_topk": ["router_topk_kernel"],
+    "router_forward": ["bn_block_stats_kernel", "router_gate_kernel", "router_select_kernel"],
+    "router_topk": ["router_select_kernel"],
     "expert": ["expert_prepare_kernel", "expert_scores_slice_kernel", "expert_gate_kernel", "expert_states_slice_kernel"],
     "expert_c5": ["bucket_clear_kernel", "bucket_histogram_kernel", "bucket_scan_kernel", "bucket_fill_kernel",
                   "expert_band_copy_kernel", "expert_scores_bucketed_kernel", "expert_gate_sorted_kernel",
