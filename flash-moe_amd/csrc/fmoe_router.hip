@@ -289,10 +289,33 @@ __global__ __launch_bounds__(kRouterWaves* kWave) __attribute__((amdgpu_waves_pe
 // List order is key index order for a half (position p = r*64 + lane), so ties at the cut go to the lowest index there;
 // among candidate sums tied at the cut the earlier candidate (lower rank in half 0) is taken.
 // ------------------------------------------------------------------------------------------------------------
-template <int R>
+__device__ inline uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int m = 1; m < kWave; m <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)v, m, kWave);
+        v = v > o ? v : o;
+    }
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
+}
+// RK = registers whose 64 * RK entries cover at least k: their smallest score bounds tau from below (k entries are at
+// least that large), the largest score of the list bounds it from above, and tau shares the leading bits the two bounds
+// share - the search starts below them (log-probabilities of one token typically share the sign, the exponent and a
+// few mantissa bits: about 22 of the 32 steps remain).  A padding entry (key 0) among those registers just gives the
+// bound 0.
+template <int R, int RK>
 __device__ inline uint32_t kth_largest_score(const uint64_t (&key)[R], int k) {
-    uint32_t tau = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
+    uint32_t hi = 0u, lo_inv = 0u;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const uint32_t s = (uint32_t)(key[r] >> 32);
+        hi = hi > s ? hi : s;
+        if (r < RK) lo_inv = lo_inv > ~s ? lo_inv : ~s;        // max of the complements = complement of the min
+    }
+    hi = wave_max_u32(hi);
+    const uint32_t lo = ~wave_max_u32(lo_inv);
+    const int bits = 32 - __builtin_clz((hi ^ lo) | 1u);         // low bits in which the bounds may differ
+    uint32_t tau = bits >= 32 ? 0u : (hi >> bits) << bits;
+    for (int bit = bits - 1; bit >= 0; --bit) {
         const uint32_t trial = tau | (1u << bit);
         int count = 0;
 #pragma unroll
@@ -311,7 +334,7 @@ __device__ inline int lanes_below(uint64_t mask) {
 template <int R, int RK>
 __device__ inline void select_topk_sorted(const uint64_t (&key)[R], int k, uint64_t* slots, uint64_t (&best)[RK], int lane) {
     constexpr int KP = RK * kWave;
-    const uint32_t tau = kth_largest_score<R>(key, k);
+    const uint32_t tau = kth_largest_score<R, RK>(key, k);
     int base = 0;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
