@@ -7,8 +7,10 @@ A step is one forward pass of the FlashMoE block (README configuration: bf16, ba
 hidden 1024, intermediate 4096, 16384 experts, top-64, norm_topk_prob False) over one synthetic batch
 that is already resident in HBM.  The last line printed is one JSON object:
 
-  value          tokens/s of the whole block (4096 tokens / mean step time over K steps)
-  stages         mean duration of each launch of the block, measured with HIP events on the launch stream
+  value          tokens/s of the whole block: 4096 tokens / ms_per_step, the median over the K timed steps of the HIP-event
+                 time of one step (step_ms has min / median / max / mean; wall_ms_per_step is the host clock over the K steps)
+  stages_us      median duration of each C-ABI call of the block, one HIP-event pair per call on the launch stream
+                 (stages_spread_us: min / median / max / mean)
   roofline       the slowest C-ABI call of the block (its kernels are named in `launches`) against the roofline
                  that bounds it; rooflines_all has every call
   expert_c3      the routed-expert kernel alone on its own benchmark shape (16384 tokens), as HBM GB/s
@@ -67,20 +69,32 @@ def synthetic_block(cfg, dtype, device):
     return m.to(device=device, dtype=dtype), x.to(device=device, dtype=dtype)
 
 
-def event_time_ms(fn, iters, warmup=3):
-    """Mean duration of fn() over `iters` back-to-back calls, from HIP events on the current stream."""
+def event_times_ms(fn, iters, warmup=3):
+    """Duration of each of `iters` back-to-back calls of fn(), from one HIP-event pair per call on the current stream
+    (the calls are queued without host synchronisation in between; one synchronisation at the end)."""
     import torch
 
     for _ in range(warmup):
         fn()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
     torch.cuda.synchronize()
-    start.record()
-    for _ in range(iters):
+    for start, stop in pairs:
+        start.record()
         fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) / iters
+        stop.record()
+    torch.cuda.synchronize()
+    return [start.elapsed_time(stop) for start, stop in pairs]
+
+
+def spread(times_ms, scale=1e3, digits=2):
+    """min / median / max / mean of a list of durations (ms), scaled (default: to microseconds)."""
+    return dict(min=round(min(times_ms) * scale, digits), median=round(statistics.median(times_ms) * scale, digits),
+                max=round(max(times_ms) * scale, digits), mean=round(statistics.fmean(times_ms) * scale, digits))
+
+
+def event_time_ms(fn, iters, warmup=3):
+    """Median duration of fn() over `iters` back-to-back calls (one HIP-event pair per call)."""
+    return statistics.median(event_times_ms(fn, iters, warmup))
 
 
 def expert_bytes(T, H, K, touched, elt):
@@ -180,7 +194,7 @@ LAUNCHES = {
 }
 
 
-def roofline_entry(name, ms, w, traffic, launches=None):
+def roofline_entry(name, ms, w, traffic, launches=None, spread_us=None):
     if w["bound"] == "hbm":
         achieved = w["bytes"] / (ms * 1e-3) / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
@@ -190,6 +204,9 @@ def roofline_entry(name, ms, w, traffic, launches=None):
     entry = dict(kernel=name, launches=LAUNCHES.get(launches or name, [name]), bound=w["bound"], achieved=round(achieved, 2),
                  peak=peak, unit=unit, frac=round(achieved / peak, 4), avg_launch_us=round(ms * 1e3, 2),
                  algorithmic=w.get("bytes", w.get("flops")), traffic=traffic)
+    if spread_us is not None:
+        entry["median_launch_us"], entry["min_launch_us"], entry["max_launch_us"] = (spread_us["median"], spread_us["min"],
+                                                                                      spread_us["max"])
     if w["bound"] == "hbm" and "flops" in w:
         # a contraction below the MFMA ridge: the matrix-core fraction next to the binding (HBM) one
         tf = w["flops"] / (ms * 1e-3) / 1e12
@@ -469,28 +486,38 @@ def main():
     m, x = synthetic_block(C4, dtype, "cuda:0")
     T = C4["batch"] * C4["seq"]
 
+    # K timed steps between two device synchronisations; inside, one HIP-event pair per step on the launch stream
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     with torch.no_grad():
         for _ in range(args.warmup):
             m(x)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for start, stop in pairs:
+            start.record()
             m(x)
+            stop.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    log(f"block: {ms_per_step:.3f} ms/step -> {T / ms_per_step * 1e3:.0f} tokens/s")
+    step_ms = [start.elapsed_time(stop) for start, stop in pairs]
+    wall_ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = statistics.median(step_ms)
+    log(f"block: median {ms_per_step:.4f} ms/step (min {min(step_ms):.4f}, max {max(step_ms):.4f}; host clock over the "
+        f"{args.steps} steps {wall_ms_per_step:.4f}) -> {T / ms_per_step * 1e3:.0f} tokens/s")
 
     # per-stage durations (HIP events on the launch stream), kernels launched through the C ABI
     fns, work, keep = stage_kernels(m, x)
     iters = max(20, min(200, args.steps))
     stages = {}
     times = {}
+    stage_spread = {}
     for name, fn in fns.items():
-        times[name] = event_time_ms(fn, iters)
-        stages[name] = round(times[name] * 1e3, 2)
-    log("stage durations (us):", stages)
-    rooflines = {n: roofline_entry(n, times[n], work[n], measured_traffic(n, "c4")) for n in fns}
+        per_call = event_times_ms(fn, iters)
+        times[name] = statistics.fmean(per_call)          # the roofline entries use the average launch duration
+        stage_spread[name] = spread(per_call)
+        stages[name] = stage_spread[name]["median"]
+    log("stage durations (us, min / median / max / mean):", stage_spread)
+    rooflines = {n: roofline_entry(n, times[n], work[n], measured_traffic(n, "c4"), spread_us=stage_spread[n]) for n in fns}
     # router_topk is part of router_forward: it is listed, but only whole launches compete for "dominant"
     dominant = max((n for n in times if n != "router_topk"), key=times.get)
 
@@ -502,6 +529,10 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
+        # ms_per_step is the median over the K steps of the HIP-event time of one step; wall_ms_per_step is the host clock
+        # between the two synchronisations divided by K
+        "step_ms": spread(step_ms, scale=1.0, digits=4),
+        "wall_ms_per_step": round(wall_ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -513,6 +544,7 @@ def main():
                    "top_k": C4["top_k"]},
         "roofline": rooflines[dominant],
         "stages_us": stages,
+        "stages_spread_us": stage_spread,
         # the block's own launches: the stages without the stand-alone top-k and without the expert op's id -> offset
         # pass (inside the block the router writes the offsets); what is left of ms_per_step is launch gaps
         "stages_sum_us": round(sum(v for k, v in stages.items() if k != "router_topk"), 2),

@@ -925,7 +925,9 @@ bool rows_possible(int H, size_t elt) { return (size_t)H * elt <= (size_t)8 * kW
 // The sweep needs 16-bit rows of whole 128-byte bands, at most 256 pairs per token, ids below 2^22 and lists below 4 GiB.
 bool sweep_possible(int64_t T_, int H, int64_t E, int K, size_t elt) {
     const int64_t padded = (T_ + kSweepTokens - 1) / kSweepTokens * kSweepTokens;
-    return elt == 2 && (H * elt) % 128 == 0 && K <= kSweepMaxTopK && E <= (1ll << 22) && padded * K * 4 < (int64_t)kBadOffset;
+    // keys are expert << 10 | token in owner << 8 | k with 0xFFFFFFFF for "no expert": E stays below 2^22 so that no pair
+    // can encode to the sentinel and the sweep's `expert < E` test rejects it
+    return elt == 2 && (H * elt) % 128 == 0 && K <= kSweepMaxTopK && E < (1ll << 22) && padded * K * 4 < (int64_t)kBadOffset;
 }
 
 // Band width: as wide as lets the band of all tokens stay in one XCD's L2 (about 2 MiB of its 4), at least 128 bytes.
@@ -1055,11 +1057,12 @@ bool slices_chosen(int64_t T_, int H, int64_t E, int K, size_t elt) {
 // 10-25 % ahead of whole-row gathers; 8 pairs per expert, 15 % behind): below that the rows are better gathered whole, straight
 // from HBM.
 bool buckets_pay(int64_t T_, int64_t E, int K) { return !slices_pay(T_, E, K) && T_ * K >= (1ll << 16) && T_ * K >= 12 * E; }
-int choose_schedule(int algo, int64_t T_, int H, int64_t E, int K, size_t elt) {
+int choose_schedule(int algo, int64_t T_, int H, int64_t E, int K, size_t elt, bool scored = true) {
     if (K == 0) return FMOE_EXPERT_ROWS;
     if (algo != FMOE_EXPERT_AUTO) return algo;
     if (slices_chosen(T_, H, E, K, elt)) return FMOE_EXPERT_SLICES;
-    if (buckets_pay(T_, E, K) && bucketed_possible(T_, E, H, K, elt)) return FMOE_EXPERT_BUCKETS;
+    // grouping by expert serves the score phase; an op without scores (product-key memory) has nothing to group
+    if (scored && buckets_pay(T_, E, K) && bucketed_possible(T_, E, H, K, elt)) return FMOE_EXPERT_BUCKETS;
     return FMOE_EXPERT_ROWS;
 }
 
@@ -1130,6 +1133,15 @@ extern "C" size_t fmoe_expert_workspace_bytes(int64_t num_tokens, int hidden, in
     return fmoe_expert_workspace_bytes_algo(num_tokens, hidden, num_experts, top_k, dtype, FMOE_EXPERT_AUTO);
 }
 
+extern "C" size_t fmoe_pkm_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype) {
+    using namespace fmoe;
+    if (num_tokens <= 0 || hidden <= 0 || num_experts <= 0 || top_k <= 0 || !dtype_ok(dtype)) return 0;
+    const size_t elt = dtype_size(dtype);
+    return choose_schedule(FMOE_EXPERT_AUTO, num_tokens, hidden, num_experts, top_k, elt, false) == FMOE_EXPERT_SLICES
+               ? plan_slices(num_tokens, hidden, num_experts, top_k, elt).bytes
+               : 0;
+}
+
 namespace fmoe {
 namespace {
 
@@ -1158,7 +1170,7 @@ int expert_dispatch(const char* who, int act, const void* x, const void* down, c
                  (long long)(num_tokens * top_k));
     hipStream_t s = (hipStream_t)stream;
     const size_t elt = dtype_size(dtype);
-    const int schedule = choose_schedule(algo, num_tokens, hidden, num_experts, top_k, elt);
+    const int schedule = choose_schedule(algo, num_tokens, hidden, num_experts, top_k, elt, act != kActNone);
     FMOE_REQUIRE(schedule != FMOE_EXPERT_SLICES || slices_possible(num_experts, hidden, elt), FMOE_ERR_UNSUPPORTED,
                  "%s: tables of 4 GiB or more cannot use the column-slice schedule", who);
     FMOE_REQUIRE(schedule != FMOE_EXPERT_BUCKETS || bucketed_possible(num_tokens, num_experts, hidden, top_k, elt),

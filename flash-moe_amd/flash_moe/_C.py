@@ -52,6 +52,7 @@ SIGNATURES = {
     "fmoe_mlp_gate_up_save": (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp]),
     "fmoe_mlp_down": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp, _vp]),
     "fmoe_peer_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
+    "fmoe_pkm_workspace_bytes": (_sz, [_i64, _int, _i64, _int, _int]),
     "fmoe_pkm_forward": (_int, [_vp, _vp, _vp, _i64, _int, _i64, _int, _int, _vp, _vp, _sz, _vp]),
     "fmoe_router_topk_backward": (_int, [_vp, _vp, _i64, _int, _int, _int, _vp, _vp]),
     "fmoe_route_backward": (_int, [_vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _vp, _vp]),

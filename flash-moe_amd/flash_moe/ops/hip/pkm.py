@@ -24,7 +24,7 @@ def pkm_forward(values, routing_weights, indices) -> torch.Tensor:
     (num_experts, hidden), (num_tokens, top_k), code = v.shape, idx.shape, _C.dtype_code(v.dtype)
     out = torch.empty((num_tokens, hidden), device=dev, dtype=v.dtype)
     L = _C.lib()
-    ws_bytes = L.fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, code)
+    ws_bytes = L.fmoe_pkm_workspace_bytes(num_tokens, hidden, num_experts, top_k, code)
     ws = torch.empty(max(ws_bytes, 1), device=dev, dtype=torch.uint8)
     with torch.cuda.device(dev):
         status = L.fmoe_pkm_forward(_C.ptr(v), _C.ptr(w), _C.ptr(idx), num_tokens, hidden, num_experts, top_k, code, _C.ptr(out),

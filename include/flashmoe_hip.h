@@ -119,7 +119,9 @@ int fmoe_router_forward_split(const void* x, const void* sub_keys, void* running
  * counterpart in the reference.  The scratch the call needs (batch-norm partials, mean and 1/std: about 6 MiB) is a
  * static array in device memory, one copy per GPU for the life of the process, so hidden is limited to 2048
  * (FMOE_ERR_UNSUPPORTED beyond) and two calls that overlap on one GPU (different streams or threads) race on it.
- * The call itself allocates and frees nothing; the device the stream belongs to must be the current device. */
+ * The call itself allocates and frees nothing; the device the stream belongs to must be the current device.  The first call
+ * on a device asks the runtime for the scratch's address and the device geometry (host-side queries, no stream work):
+ * make one call outside any capture before capturing the entry point into a graph. */
 int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running_mean, void* running_var,
                                 int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
                                 int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
@@ -144,7 +146,8 @@ int fmoe_router_forward_noalloc(const void* x, const void* gate_w, void* running
  * schedule (FMOE_ERR_UNSUPPORTED when a call can take none of them, or when the forced one does not apply):
  *   rows     rows of at most 8192 bytes (hidden <= 4096 for the 16-bit dtypes, 2048 for fp32)
  *   slices   each table below 4 GiB (rows are addressed with 32-bit byte offsets)
- *   buckets  rows a multiple of 128 bytes; x and each table below 4 GiB; T*K < 2^31 - 4096; T < 2^24
+ *   buckets  rows a multiple of 128 bytes; x and each table below 4 GiB; T*K < 2^31 - 4096; T < 2^24 (its second
+ *            phase sweeps the experts when the dtype is 16-bit, K <= 256 and E < 2^22; else it gathers whole rows)
  * fmoe_expert_forward picks slices when E*128 bytes fit twice the L2 of one XCD and there are at least 65536 pairs, or
  * when the rows are too long for the row schedule; else buckets when there are at least 65536 pairs and 12 pairs per
  * expert (each table row then serves enough pairs to pay for the grouping) and its limits hold; else rows.  So any
@@ -257,8 +260,12 @@ int fmoe_block_forward(const void* x, const void* gate_proj_w, const void* up_pr
  *
  * PKM, triton_pkm_func / pkm_forward (flash_moe/ops/triton/pkm.py:195-200, 123-174; eager form tests/test_pkm.py:9-20):
  *   out[t] = sum_k w[t,k] * values[idx[t,k]]
- * Both take a workspace of fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, dtype) bytes.
+ * PEER takes a workspace of fmoe_expert_workspace_bytes(num_tokens, hidden, num_experts, top_k, dtype) bytes.  PKM has no
+ * score phase, so it never groups pairs by expert: it takes fmoe_pkm_workspace_bytes(...) bytes (the column-slice
+ * workspace when the slices are chosen, else nothing).
  */
+size_t fmoe_pkm_workspace_bytes(int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype);
+
 int fmoe_peer_forward(const void* x, const void* down, const void* up, const void* routing_weights, const int64_t* indices,
                       int64_t num_tokens, int hidden, int64_t num_experts, int top_k, int dtype, void* out, void* workspace,
                       size_t workspace_bytes, void* stream);

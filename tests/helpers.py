@@ -45,3 +45,4 @@ def assert_mostly_close(got, ref, dtype, what="", max_outliers=1e-4):
     assert bad <= max_outliers, f"{what}: {bad:.2e} of the elements outside rtol=atol={tol}"
     assert rel_fro(g, r) <= FRO_TOL[dtype], f"{what}: relative Frobenius error {rel_fro(g, r):.3e}"
     assert max_rel_to_scale(g, r) <= 2 * tol, f"{what}: max|diff|/max|ref| = {max_rel_to_scale(g, r):.3e}"
+    return bad

@@ -114,6 +114,13 @@ def test_expert_argument_checks():
     assert lib.fmoe_expert_workspace_bytes_algo(64, 1024, 16384, 8, _C.BF16, _C.EXPERT_SLICES) > 0
     assert lib.fmoe_expert_workspace_bytes_algo(4096, 1024, 16384, 64, _C.BF16, _C.EXPERT_ROWS) == 0
     assert lib.fmoe_expert_workspace_bytes_algo(4096, 1024, 16384, 64, _C.BF16, _C.EXPERT_AUTO) == sliced
+    # a product-key memory has no score phase: it never takes the bucketed plan's workspace (the reference's PKM
+    # benchmark shape, tests/test_pkm.py: 16384 tokens, top-2500, would ask for gigabytes of partial scores there)
+    assert lib.fmoe_pkm_workspace_bytes(4096, 1024, 16384, 64, _C.BF16) == sliced
+    assert lib.fmoe_pkm_workspace_bytes(32768, 2048, 262144, 128, _C.BF16) == 0
+    assert lib.fmoe_pkm_workspace_bytes(16384, 1024, 1 << 20, 2500, _C.BF16) == 0 < lib.fmoe_expert_workspace_bytes(
+        16384, 1024, 1 << 20, 2500, _C.BF16)
+    assert lib.fmoe_pkm_workspace_bytes(0, 1024, 16, 4, _C.BF16) == 0 and lib.fmoe_pkm_workspace_bytes(4, 1024, 16, 4, 9) == 0
 
 
 def test_mlp_argument_checks():

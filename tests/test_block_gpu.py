@@ -37,10 +37,11 @@ def stagewise_check(m, w, x, K, norm, dtype):
     w.running_mean.zero_(); w.running_var.fill_(1.0)
     ref = orc.block_forward(x, w, K, norm_topk_prob=norm, training=True, routing_fp32=True, token_chunk=256)
     assert_output_close(logits, ref["router_logits"], dtype, "router_logits")
+    outliers = 0.0
     if dtype == torch.float32:
         assert_output_close(y, ref["y"], dtype, "block output")
     else:
-        assert_mostly_close(y, ref["y"], dtype, "block output vs same-dtype oracle")
+        outliers = assert_mostly_close(y, ref["y"], dtype, "block output vs same-dtype oracle")
     # running statistics follow nn.BatchNorm1d
     torch.testing.assert_close(m.router_norm.running_mean.float().cpu(), w.running_mean.float(), rtol=2e-2, atol=1e-3)
     torch.testing.assert_close(m.router_norm.running_var.float().cpu(), w.running_var.float(), rtol=2e-2, atol=1e-3)
@@ -78,7 +79,7 @@ def stagewise_check(m, w, x, K, norm, dtype):
     # HIP path's two roundings (the [T,I] activation and the result) remain, so the bar holds everywhere
     y64 = orc.mlp_forward(x.view(-1, H).double(), w.gate_proj.double(), w.up_proj.double(), w.down_proj.double()) + e_hip.double()
     assert_output_close(y.view(-1, H), y64.to(dtype), dtype, "block output vs float64 oracle")
-    return same
+    return dict(overlap_fp32_routing=same, outlier_fraction=outliers, indices=idx_cpu)
 
 
 @pytest.mark.parametrize("norm", [False, True])
@@ -94,7 +95,19 @@ def test_block_c4_shape_fewer_tokens(dtype):
     # C4 weights (H=1024, I=4096, E=16384, K=64) on 512 tokens so that the CPU oracle finishes in seconds
     m, w = build(1024, 4096, 16384, 64, False, dtype)
     x = torch.randn(1, 512, 1024, generator=torch.Generator().manual_seed(0)).to(dtype)
-    stagewise_check(m, w, x, 64, False, dtype)
+    res = stagewise_check(m, w, x, 64, False, dtype)
+    # How far the expert sets are from the reference's literal 16-bit routing (logits, log-softmax and pair sums all
+    # rounded to the dtype, where many sums tie and the choice among ties is the library's): measured, and bounded
+    # from below so that a regression of the routing shows.
+    w.running_mean.zero_(); w.running_var.fill_(1.0)
+    literal = orc.block_forward(x, w, 64, norm_topk_prob=False, training=True, routing_fp32=False, token_chunk=256)
+    hit = torch.tensor([len(set(a.tolist()) & set(b.tolist())) for a, b in zip(res["indices"], literal["indices"])]).float()
+    overlap_literal = (hit / 64).mean().item()
+    print(f"\n[{dtype}] 512 tokens of C4: expert-set overlap with the oracle's fp32 routing {res['overlap_fp32_routing']:.4f}, "
+          f"with its literal 16-bit routing {overlap_literal:.4f}; elements of y outside rtol = atol = 2e-2 against the "
+          f"same-dtype oracle: {res['outlier_fraction']:.2e} (budget 1e-4)")
+    assert res["outlier_fraction"] <= 1e-4
+    assert overlap_literal > 0.5, overlap_literal
 
 
 def test_block_c4_full_size_properties():

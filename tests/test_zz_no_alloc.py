@@ -58,3 +58,45 @@ def test_noalloc_router_rejects_sizes_beyond_its_scratch():
     a = _C.ptr(x)
     status = L.fmoe_router_forward_noalloc(a, a, a, a, a, _C.F32, 1, 0.1, 1e-5, 4, 4096, 8, 2, _C.BF16, 0, a, a, a, a, a, None)
     assert status == -5 and b"2048" in L.fmoe_last_error()
+
+
+def test_noalloc_router_in_a_hip_graph_after_one_warm_up_call():
+    """The first call on a device looks up the address of the static scratch and the device geometry (host-side queries,
+    not stream work), so one eager call precedes the capture; after it the entry point only launches kernels, and every
+    replay of a graph that holds it equals the eager workspace entry point on the same input."""
+    dtype, T, H, nk, K = torch.bfloat16, 1024, 512, 64, 32
+    g = torch.Generator().manual_seed(5)
+    dev = torch.device("cuda")
+    w = (torch.randn(2 * nk, H, generator=g) * 0.02).to(dtype).cuda()
+    static_x = torch.randn(T, H, generator=g).to(dtype).cuda()
+    _route("noalloc", static_x, w, nk, K, False, True)                      # the warm-up call
+    rm, rv = torch.zeros(H, device=dev), torch.ones(H, device=dev)
+    nbt = torch.zeros(1, device=dev, dtype=torch.int64)
+    logits = torch.empty(T, 2 * nk, device=dev, dtype=dtype)
+    logits32 = torch.empty(T, 2 * nk, device=dev, dtype=torch.float32)
+    scores = torch.empty(T, K, device=dev, dtype=torch.float32)
+    indices = torch.empty(T, K, device=dev, dtype=torch.int64)
+    gates = torch.empty(T, K, device=dev, dtype=dtype)
+    L = _C.lib()
+
+    def call():
+        _C.check(L.fmoe_router_forward_noalloc(_C.ptr(static_x), _C.ptr(w), _C.ptr(rm), _C.ptr(rv), _C.ptr(nbt), _C.F32, 0, 0.1,
+                                               1e-5, T, H, nk, K, _C.BF16, 1, _C.ptr(logits), _C.ptr(logits32), _C.ptr(scores),
+                                               _C.ptr(indices), _C.ptr(gates), _C.current_stream(dev)), "noalloc in capture")
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for step in range(3):
+        new_x = torch.randn(T, H, generator=torch.Generator().manual_seed(20 + step)).to(dtype).cuda()
+        ref = _route("workspace", new_x, w, nk, K, False, True)              # eager work between the replays
+        static_x.copy_(new_x)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b, name in zip((logits, logits32, scores, indices, gates), ref, ("logits", "logits32", "scores", "indices", "gates")):
+            assert torch.equal(a, b), f"replay {step}: {name} differs"
