@@ -359,31 +359,25 @@ __device__ inline void select_topk_sorted(const uint64_t (&key)[R], int k, uint6
     bitonic_sort<RK, true>(best, lane);
 }
 
+// The candidate pairs (rank in half 0) | (rank in half 1) << 8, listed by rank in half 0: the list depends on top_k only,
+// so the host writes it and it travels as a kernel argument (at most 64 * 11 entries for top_k <= 128).
+constexpr int kSelectMaxCand = 11 * kWave;
+struct CandidateTable { uint16_t pair[kSelectMaxCand]; };
+
 template <typename T, typename TG, int RK, int RH, int RC, bool FROM_LOGITS>
 __global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
     const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
     int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets,
-    uint32_t row_bytes) {
+    uint32_t row_bytes, const CandidateTable table) {
     constexpr int KP = RK * kWave;
+    static_assert(RC * kWave <= kSelectMaxCand, "candidate table");
     __shared__ uint16_t cand[RC * kWave];
     __shared__ float half_score[kRouterWaves][2][KP];
     __shared__ uint32_t half_index[kRouterWaves][2][KP];
     __shared__ uint64_t slot[kRouterWaves][KP];
 
-    // candidate table, as in router_topk_kernel
-    {
-        uint32_t* row_len = &half_index[0][0][0];
-        for (int i = threadIdx.x; i < top_k; i += blockDim.x) row_len[i] = (uint32_t)(top_k / (i + 1));
-        __syncthreads();
-        for (int i = threadIdx.x; i < top_k; i += blockDim.x) {
-            int off = 0;
-            for (int q = 0; q < i; ++q) off += (int)row_len[q];
-            const int n = (int)row_len[i];
-            for (int j = 0; j < n; ++j) cand[off + j] = (uint16_t)(i | (j << 8));
-        }
-        __syncthreads();
-    }
-
+    for (int i = (int)threadIdx.x; i < RC * kWave; i += (int)blockDim.x) cand[i] = table.pair[i];
+    __syncthreads();
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
     const int64_t waves_total = (int64_t)gridDim.x * kRouterWaves;
@@ -614,7 +608,14 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
     // lists that fit the registers of a wave take the threshold selection
 #define FMOE_LAUNCH_SELECT(RK_, RH_, RC_)                                                                              \
     hipLaunchKernelGGL((router_select_kernel<T, TG, RK_, RH_, RC_, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, \
-                       T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes)
+                       T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes, table)
+    CandidateTable table;
+    if (K <= 128 && nk <= 512) {
+        int c = 0;
+        for (int i = 0; i < K; ++i)
+            for (int j = 0; j < K / (i + 1); ++j) table.pair[c++] = (uint16_t)(i | (j << 8));
+        for (; c < kSelectMaxCand; ++c) table.pair[c] = 0;
+    }
     if (K <= 64 && nk <= 512) {
         if (nk <= 128) FMOE_LAUNCH_SELECT(1, 2, 5);
         else FMOE_LAUNCH_SELECT(1, 8, 5);

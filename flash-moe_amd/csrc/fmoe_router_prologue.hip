@@ -12,7 +12,8 @@
 //                          staged: (x - mean) * rstd is rounded to the activation dtype exactly as a stand-alone
 //                          batch-norm would emit it, then multiplied with the gate weights with fp32 accumulation;
 //                          writes the logits in fp32 (for the routing) and in the activation dtype (the tensor the
-//                          module returns)
+//                          module returns).  With at most one tile per compute unit (4096 tokens) a workgroup is 16
+//                          waves: four groups that each take every fourth k-tile and add their accumulators at the end
 //   router_topk_kernel     (fmoe_router.hip)
 // fp32 activations (a parity configuration, not tuned): bn_partial_kernel per (row block, 512-column strip),
 // bn_finalize_kernel per column, router_gate_f32_kernel, router_topk_kernel.
@@ -367,20 +368,28 @@ constexpr int kGateMaxK = 8192;     // mean / rstd of all k are staged in LDS on
 
 // split != 0: half h of the outputs (columns [h*N/2, (h+1)*N/2)) scores only half h of the normalised activations,
 // w is [N, K/2]: the product-key form in which each sub-key table sees its own half of the query (a block-diagonal gate).
-template <typename T>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w, GateStats st,
+// KG > 1: the k-tiles are dealt to KG groups of four waves (group g takes k-tiles g, g + KG, ...), each with LDS tiles
+// and an accumulator of its own, and the groups' accumulators are added in group order through LDS at the end.  With
+// 256 tiles for 256 compute units a tile's k loop is a chain of global-load latencies; KG = 4 runs four of them side by
+// side on the same compute unit.  The result depends on KG (another summation order), not on anything else.
+template <typename T, int KG>
+__global__ __launch_bounds__(256 * KG) __attribute__((amdgpu_waves_per_eu(4, 4))) void router_gate_kernel(const T* __restrict__ x, const T* __restrict__ w, GateStats st,
                                                           float* __restrict__ logits32, T* __restrict__ logits, int M, int N,
                                                           int K_full, int tiles_m, int tiles_n, int split, int xcds) {
     using Frag = typename Mfma32<T>::Frag;
     constexpr int BM = 64, BN = 64, CH = 2;   // CH = 16-byte packets per thread per tile and operand
-    constexpr int D = kGatePrefetch;
-    __shared__ __attribute__((aligned(16))) T As[BM * kTileK];
-    __shared__ __attribute__((aligned(16))) T Bs[BN * kTileK];
+    constexpr int D = KG > 1 ? 4 : kGatePrefetch;
+    constexpr int THREADS = 256 * KG;
+    __shared__ __attribute__((aligned(16))) T tiles[KG][2][BM * kTileK];
     extern __shared__ __attribute__((aligned(16))) float stats[];   // [2][Kpad]: mean, rstd
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, xcds, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid_all = (int)threadIdx.x;
+    const int grp = __builtin_amdgcn_readfirstlane(tid_all / 256);
+    const int tid = tid_all % 256, lane = tid & 63, wave = tid >> 6;
+    T* As = tiles[grp][0];
+    T* Bs = tiles[grp][1];
     const int wm = wave >> 1, wn = wave & 1;
     const int ch = tid % kTileChunks;          // this thread's packet column inside a k-tile: the same for all its packets
     const int row0 = tid / kTileChunks;        // rows row0 and row0 + 32
@@ -390,9 +399,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int k_off = (split && n0 >= N / 2) ? K : 0;
     const int k_tiles = (K + kTileK - 1) / kTileK;
     const int kpad = k_tiles * kTileK;
+    const int steps = (k_tiles + KG - 1) / KG;         // k-tile of step s in this group: grp + s * KG
     u32x4_t ra[D][CH], rb[D][CH];
 
-    auto load_global = [&](int kt, int slot) {
+    auto load_global = [&](int step, int slot) {
+        const int kt = grp + step * KG;
         const int gk = kt * kTileK + ch * 8;
         const bool k_ok = kt < k_tiles && gk < K;
 #pragma unroll
@@ -402,8 +413,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             rb[slot][it] = (gn < N && k_ok) ? *reinterpret_cast<const u32x4_t*>(w + (int64_t)gn * K + gk) : zero4;
         }
     };
-    auto store_lds = [&](int kt, int slot) {
-        const float* mu = stats + kt * kTileK + ch * 8;
+    auto store_lds = [&](int step, int slot) {
+        const int kt = grp + step * KG;
+        const float* mu = stats + (kt < k_tiles ? kt : 0) * kTileK + ch * 8;     // a step beyond the range multiplies zeros
         const float* rs = mu + kpad;
         float m8[8], r8[8];
 #pragma unroll
@@ -413,7 +425,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }
 #pragma unroll
         for (int it = 0; it < CH; ++it) {
-            *reinterpret_cast<u32x4_t*>(&As[swizzled_offset(row0 + it * 32, ch)]) = normalise16<T>(ra[slot][it], m8, r8);
+            *reinterpret_cast<u32x4_t*>(&As[swizzled_offset(row0 + it * 32, ch)]) =
+                kt < k_tiles ? normalise16<T>(ra[slot][it], m8, r8) : zero4;
             *reinterpret_cast<u32x4_t*>(&Bs[swizzled_offset(row0 + it * 32, ch)]) = rb[slot][it];
         }
     };
@@ -421,28 +434,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
     const int frow = lane & 31, fhalf = lane >> 5;
+    // with k groups the operands of the first steps are requested before the statistics are combined: the two latencies overlap
+    // (of the first two steps: the block statistics need the other registers)
+    if (KG > 1) {
+#pragma unroll
+        for (int d = 0; d < 2; ++d) load_global(d, d);
+    }
     // mean and 1/std of this tile's k range into LDS.  One column of tiles per k range also stores them (for a backward
     // pass) and updates the running statistics: tile row (i / 64) mod tiles_m takes column i, so every column is written
-    // by exactly one workgroup.  Two columns per thread and round: all their block statistics are loaded together (one
+    // by exactly one workgroup.  CPT columns per thread and round: all their block statistics are loaded together (one
     // memory round trip per round), before the operand prefetch below claims its registers.
     {
-        constexpr int CPT = 2;
+        constexpr int CPT = KG > 1 ? 1 : 2;
         const bool keeper = tn == (k_off ? tiles_n / 2 : 0);
-        if (blockIdx.x == 0 && tid == 0 && st.training && !st.ready && st.num_batches_tracked != nullptr) *st.num_batches_tracked += 1;
+        if (blockIdx.x == 0 && tid_all == 0 && st.training && !st.ready && st.num_batches_tracked != nullptr) *st.num_batches_tracked += 1;
         const float n = (float)st.num_tokens;
         const float full = (float)st.rows_per_block;
         const float last = (float)(st.num_tokens - (int64_t)(st.row_blocks - 1) * st.rows_per_block);
-        for (int i0 = tid; st.ready && i0 < kpad; i0 += 256) {
+        for (int i0 = tid_all; st.ready && i0 < kpad; i0 += THREADS) {
             stats[i0] = i0 < K ? st.mean_rstd[k_off + i0] : 0.0f;
             stats[kpad + i0] = i0 < K ? st.mean_rstd[K_full + k_off + i0] : 0.0f;
         }
-        for (int i0 = tid; !st.ready && i0 < kpad; i0 += 256 * CPT) {
+        for (int i0 = tid_all; !st.ready && i0 < kpad; i0 += THREADS * CPT) {
             float mean[CPT], var[CPT], m2[CPT];
             if (st.training) {
                 float mb[CPT][kFoldMaxRowBlocks], m2b[CPT][kFoldMaxRowBlocks];
 #pragma unroll
                 for (int u = 0; u < CPT; ++u) {
-                    const int i = i0 + u * 256;
+                    const int i = i0 + u * THREADS;
                     const float* pc = st.partial + k_off + (i < K ? i : 0);
 #pragma unroll
                     for (int b = 0; b < kFoldMaxRowBlocks; ++b) {
@@ -473,7 +492,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             } else {
 #pragma unroll
                 for (int u = 0; u < CPT; ++u) {
-                    const int i = i0 + u * 256;
+                    const int i = i0 + u * THREADS;
                     const int c = k_off + (i < K ? i : 0);
                     mean[u] = load_stat_rt(st.running_mean, c, st.stats_dtype);
                     var[u] = load_stat_rt(st.running_var, c, st.stats_dtype);
@@ -482,7 +501,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             }
 #pragma unroll
             for (int u = 0; u < CPT; ++u) {
-                const int i = i0 + u * 256;
+                const int i = i0 + u * THREADS;
                 if (i >= kpad) continue;
                 const int c = k_off + i;
                 const float rstd = 1.0f / sqrtf(var[u] + st.eps);
@@ -501,16 +520,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }
     }
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_global(d, d);
+    for (int d = KG > 1 ? 2 : 0; d < D; ++d) load_global(d, d);
     __syncthreads();               // stats[] visible
-    // the k loop is unrolled by D so that the register slot of a tile is a compile-time index
-    for (int kt0 = 0; kt0 < k_tiles; kt0 += D) {
+    // the step loop is unrolled by D so that the register slot of a tile is a compile-time index; every group runs every
+    // step (a step beyond its k-tiles multiplies zeros), so the barriers are reached by all waves
+    for (int s0 = 0; s0 < steps; s0 += D) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            const int kt = kt0 + d;
-            if (kt < k_tiles) {
-                store_lds(kt, d);
-                load_global(kt + D, d);        // slot d is free again
+            const int step = s0 + d;
+            if (step < steps) {
+                store_lds(step, d);
+                load_global(step + D, d);        // slot d is free again
                 __syncthreads();
 #pragma unroll
                 for (int ks = 0; ks < kTileK / 16; ++ks) {
@@ -522,6 +542,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 __syncthreads();
             }
         }
+    }
+    if (KG > 1) {
+        // groups 1 .. KG-1 hand their accumulators over through the tile memory; group 0 adds them in group order
+        float* red = reinterpret_cast<float*>(&tiles[0][0][0]);
+        static_assert(KG == 1 || (KG - 1) * BM * BN * sizeof(float) <= sizeof(tiles), "reduction fits the tile memory");
+        if (grp > 0) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[(grp - 1) * BM * BN + (wave * 16 + v) * kWave + lane] = acc[v];
+        }
+        __syncthreads();
+        if (grp > 0) return;
+#pragma unroll
+        for (int g = 1; g < KG; ++g)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] += red[(g - 1) * BM * BN + (wave * 16 + v) * kWave + lane];
     }
     const int col = n0 + wn * 32 + frow;
 #pragma unroll
@@ -1064,14 +1099,20 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
         st.num_batches_tracked = num_batches_tracked;
         st.mean_rstd = mean_rstd;
         const size_t stats_bytes = (size_t)((hidden + kTileK - 1) / kTileK) * kTileK * 2 * sizeof(float);
-        if (dtype == FMOE_BF16)
-            hipLaunchKernelGGL((router_gate_kernel<bf16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
-                               (const bf16_t*)x, (const bf16_t*)gate_w, st, logits32, (bf16_t*)router_logits, M, N, hidden,
-                               tiles_m, tiles_n, split_query, chip_info().xcds);
-        else
-            hipLaunchKernelGGL((router_gate_kernel<f16_t>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), stats_bytes, s,
-                               (const f16_t*)x, (const f16_t*)gate_w, st, logits32, (f16_t*)router_logits, M, N, hidden,
-                               tiles_m, tiles_n, split_query, chip_info().xcds);
+        // few tiles with a long k loop: four k groups per workgroup; many tiles already fill the chip
+        const bool k_groups = (int64_t)tiles_m * tiles_n <= chip_info().cus && (split_query ? hidden / 2 : hidden) >= 8 * kTileK;
+#define FMOE_LAUNCH_GATE(TT, KG)                                                                                            \
+    hipLaunchKernelGGL((router_gate_kernel<TT, KG>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256 * KG), stats_bytes, s,  \
+                       (const TT*)x, (const TT*)gate_w, st, logits32, (TT*)router_logits, M, N, hidden, tiles_m, tiles_n,   \
+                       split_query, chip_info().xcds)
+        if (dtype == FMOE_BF16) {
+            if (k_groups) FMOE_LAUNCH_GATE(bf16_t, 4);
+            else FMOE_LAUNCH_GATE(bf16_t, 1);
+        } else {
+            if (k_groups) FMOE_LAUNCH_GATE(f16_t, 4);
+            else FMOE_LAUNCH_GATE(f16_t, 1);
+        }
+#undef FMOE_LAUNCH_GATE
     }
     FMOE_CHECK_LAUNCH("fmoe_router_forward(gate)");
     if (top_k == 0) return FMOE_OK;
