@@ -17,6 +17,7 @@ that is already resident in HBM.  The last line printed is one JSON object:
   router_c2      the routing stage alone on the router benchmark shape: module semantics (every half scores the full
                  query) and the configuration as worded (two sub-key tables on the two halves of the query)
   block_c5       the largest block (32768 tokens, 262144 experts), with its stages and the expert op's roofline entry
+  mlp_fp32       the shared MLP of the same shape in fp32 (v_mfma_f32_32x32x2_f32) against the dense fp32 matrix peak
   cpu_baseline   the CPU restatement of the reference's eager path (oracle/) on the same block, timed on
                  this machine's host cores; cpu_baseline_c1 / cpu_baseline_c4_fp32: the reference's own CPU
                  configuration (fp32, 512 tokens) and the README block in fp32
@@ -42,6 +43,7 @@ for p in (ROOT, os.path.join(ROOT, "flash-moe_amd")):
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix
 
 C1 = dict(batch=1, seq=512, hidden=256, inter=1024, experts=1024, top_k=16, norm=False)
 C4 = dict(batch=1, seq=4096, hidden=1024, inter=4096, experts=16384, top_k=64, norm=False)
@@ -364,6 +366,25 @@ def bench_block_c5(dtype, iters):
                 mlp_TFLOPs=round(6 * T * cfg["hidden"] * cfg["inter"] / ((times["mlp_gate_up"] + times["mlp_down"]) * 1e-3) / 1e12, 1))
 
 
+def bench_mlp_fp32(iters):
+    """The C4 shared MLP in fp32: both GEMMs on v_mfma_f32_32x32x2_f32, priced against the dense fp32 matrix peak."""
+    import torch
+
+    from flash_moe.ops.hip.flash_mlp import mlp_forward
+
+    T, H, I = C4["batch"] * C4["seq"], C4["hidden"], C4["inter"]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(T, H, device="cuda", generator=g)
+    wg, wu = (torch.randn(I, H, device="cuda", generator=g) * 0.02 for _ in range(2))
+    wd = torch.randn(H, I, device="cuda", generator=g) * 0.02
+    per_call = event_times_ms(lambda: mlp_forward(x, wg, wu, wd), iters, warmup=3)
+    ms = statistics.median(per_call)
+    tf = 6.0 * T * H * I / (ms * 1e-3) / 1e12
+    return dict(workload=f"C4 shared MLP in fp32: {T} tokens, hidden {H}, intermediate {I} (gate/up + down launches)",
+                bound="mfma", dtype="f32", us=spread(per_call), achieved=round(tf, 1), peak=MFMA_FP32_PEAK_TFLOPS,
+                unit="TFLOP/s", frac=round(tf / MFMA_FP32_PEAK_TFLOPS, 4))
+
+
 def bench_backward_c4(dtype, iters):
     """Forward + backward of the C4 block through autograd (the differentiable composition of the three ops)."""
     import torch
@@ -563,6 +584,8 @@ def main():
         result["block_c5"] = bench_block_c5(dtype, 5)
         log("block C5:", result["block_c5"])
         torch.cuda.empty_cache()
+        result["mlp_fp32"] = bench_mlp_fp32(10)
+        log("mlp fp32:", result["mlp_fp32"])
         result["backward_c4"] = bench_backward_c4(dtype, 10)
         log("backward C4:", result["backward_c4"])
         torch.cuda.empty_cache()

@@ -21,6 +21,20 @@ template <> struct Mfma32<f16_t> {
     }
 };
 
+// fp32: v_mfma_f32_32x32x2_f32, D[32x32] += A[32x2] * B[2x32]; lane l supplies A[l%32][l/32] and B[l/32][l%32], same D
+// layout.  A fragment is one 16-byte LDS read like the 16-bit ones: 4 consecutive k values of the lane's row, lanes
+// 0-31 from the first 16-byte chunk of a 32-byte k-step and lanes 32-63 from the second, so instruction q of a run
+// multiplies the k pair {q, 4 + q} of the step - each of the 8 k values once.
+template <> struct Mfma32<float> {
+    using Frag = f32x4_t;
+    __device__ static f32x16_t run(Frag a, Frag b, f32x16_t c) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q], b[q], c, 0, 0, 0);
+        return c;
+    }
+};
+template <typename T> constexpr int kMfmaPerRun = sizeof(T) == 4 ? 4 : 1;   // matrix instructions per Mfma32<T>::run
+
 // Register-staged LDS tiles: rows of 64 elements (128 bytes), 16-byte chunk index XOR-ed with (row & 7).
 constexpr int kTileK = 64;
 constexpr int kTileChunks = kTileK / 8;

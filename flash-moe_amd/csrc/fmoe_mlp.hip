@@ -17,7 +17,10 @@
 // the chunk that belongs at its LDS position.  Workgroup ids are remapped so that each XCD (ids are dealt
 // round-robin over the 8 XCDs) works on a compact patch of the tile grid and shares A/B tiles in its own L2.
 //
-// Ragged shapes take gemm_nt_kernel (register-staged, bounds-checked); fp32 takes a plain FMA kernel.
+// fp32 runs the same kernel on v_mfma_f32_32x32x2_f32: an LDS row is again 128 bytes (32 values), a fragment again one
+// 16-byte read, and four matrix instructions use it.
+//
+// Ragged shapes take gemm_nt_kernel (register-staged, bounds-checked), in fp32 a plain FMA kernel.
 #include "fmoe_common.h"
 #include "fmoe_mfma.h"
 
@@ -197,16 +200,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     using Frag = typename Mfma32<T>::Frag;
     constexpr int NWAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MF = WM / 32, NF = WN / 32;
-    constexpr int CPR = BKT / 8;                    // 16-byte chunks per LDS row
+    constexpr int EPC = 16 / (int)sizeof(T);        // elements per 16-byte chunk
+    constexpr int CPR = BKT / EPC;                  // 16-byte chunks per LDS row
     constexpr int RPI = 64 / CPR;                   // rows one wave-wide DMA load covers
     constexpr int ROWS_PER_IT = NWAVES * RPI;       // rows all waves cover per DMA round
     constexpr int STAGE = (BM + BN) * BKT;          // elements per stage
-    constexpr int KSTEPS = BKT / 16;
+    constexpr int KSTEPS = BKT / (2 * EPC);         // a k-step is 32 bytes of a row: one chunk per lane half
     constexpr int ROW_SHIFT = (CPR == 8) ? 1 : 2;   // log2(rows per 256 bytes)
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
     constexpr int A_ROUNDS = BM / ROWS_PER_IT, B_ROUNDS = BN / ROWS_PER_IT;
     constexpr int DMA_PER_TILE = A_ROUNDS + B_ROUNDS;
-    static_assert(BKT == 32 || BKT == 64, "stage depth");
+    static_assert(CPR == 4 || CPR == 8, "stage depth: LDS rows of 64 or 128 bytes");
     static_assert(ROWS_PER_IT % 16 == 0 && BM % ROWS_PER_IT == 0 && BN % ROWS_PER_IT == 0, "DMA rounds");
     static_assert(EPI != kEpiSwiGLU || ((BN / 2) % ROWS_PER_IT == 0 && NF % 2 == 0), "gate/up split");
     static_assert((NSTAGE - 2) * DMA_PER_TILE < 64, "vmcnt range");
@@ -223,7 +227,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     // key does not depend on the round and one element offset per lane serves every load.
     const int lrow = lane / CPR, lp = lane % CPR;
     const int key_dma = ((wave * RPI + lrow) >> ROW_SHIFT) & (CPR - 1);
-    const uint32_t lane_off = (uint32_t)(lrow * K + ((lp ^ key_dma) << 3)) * (uint32_t)sizeof(T);   // bytes
+    const uint32_t lane_off = (uint32_t)(lrow * K + (lp ^ key_dma) * EPC) * (uint32_t)sizeof(T);   // bytes
     // A rows beyond M (a ragged last tile row) are read from row M-1 instead: one byte offset per DMA round, set per
     // tile.  What the MFMAs make of those rows is never stored (the epilogue's buffer stores are bounds-checked).
     uint32_t a_lane_off[A_ROUNDS];
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         for (int r = 0; r < A_ROUNDS; ++r) {
             int row = r * ROWS_PER_IT + wave * RPI + lrow;
             row = m0 + row < M ? row : M - 1 - m0;
-            a_lane_off[r] = (uint32_t)(row * K + ((lp ^ key_dma) << 3)) * (uint32_t)sizeof(T);
+            a_lane_off[r] = (uint32_t)(row * K + (lp ^ key_dma) * EPC) * (uint32_t)sizeof(T);
         }
         b_src0 = B0 + (int64_t)(n0 + wave * RPI) * K;
         if (EPI == kEpiSwiGLU) b_src1 = B1 + (int64_t)(n0 + wave * RPI) * K;
@@ -335,7 +339,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
             const char* next_stage = reinterpret_cast<const char*>(lds + ((kt + 1) % NSTAGE) * STAGE);
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
-                constexpr int kReads = MF + NF, kMfmas = MF * NF;
+                constexpr int kReads = MF + NF, kMfmas = MF * NF;     // kMfmas runs of kMfmaPerRun<T> instructions
                 const int nxt = ks + PF;
                 const bool reads = nxt < KSTEPS || !kLast;
                 __builtin_amdgcn_sched_barrier(0);
@@ -356,7 +360,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
                 constexpr int kPer = (kReads + kMfmas - 1) / kMfmas;
 #pragma unroll
                 for (int q = 0; q < kMfmas; ++q) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRun<T>, 0);
                     if (reads && q * kPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
                 }
             }
@@ -386,10 +390,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         // a wave whose rows all lie beyond M gets an empty descriptor: every access of it is dropped
         const int span32 = (int)(span < 0 ? 0 : (span < 0x7FFFFFFFll ? span : 0x7FFFFFFFll));
         auto c_rsrc = __builtin_amdgcn_make_buffer_rsrc(C + wave_off, 0, span32, 0x00020000);
-        auto store_elem = [&](int uni_bytes, float value) {
-            const T t = Elem<T>::from_f32(value);
-            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, t), c_rsrc, lane_bytes, uni_bytes, 0);
+        auto store_to = [&](auto rsrc, int uni_bytes, float value) {
+            if constexpr (sizeof(T) == 4) {
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, value), rsrc, lane_bytes, uni_bytes, 0);
+            } else {
+                const T t = Elem<T>::from_f32(value);
+                __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, t), rsrc, lane_bytes, uni_bytes, 0);
+            }
         };
+        auto store_elem = [&](int uni_bytes, float value) { store_to(c_rsrc, uni_bytes, value); };
+        // 16-bit outputs round once, so the fast reciprocal's last-bit error is invisible; fp32 divides
+        auto silu = [](float v) { return sizeof(T) == 4 ? silu_f32(v) : silu_fast_f32(v); };
         if (EPI == kEpiSwiGLU) {
             if (R != nullptr) {
                 // keep the gate and up products for a backward pass: planes [0] and [1] of a [2, M, N] buffer
@@ -403,9 +414,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int uni = ((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T);
-                            const T g = Elem<T>::from_f32(acc[i][j][v]), u = Elem<T>::from_f32(acc[i][j + NF / 2][v]);
-                            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, g), g_rsrc, lane_bytes, uni, 0);
-                            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, u), u_rsrc, lane_bytes, uni, 0);
+                            store_to(g_rsrc, uni, acc[i][j][v]);
+                            store_to(u_rsrc, uni, acc[i][j + NF / 2][v]);
                         }
             }
 #pragma unroll
@@ -415,7 +425,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
                         store_elem(((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T),
-                                   silu_fast_f32(acc[i][j][v]) * acc[i][j + NF / 2][v]);
+                                   silu(acc[i][j][v]) * acc[i][j + NF / 2][v]);
         } else {
             auto r_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(R != nullptr ? R + wave_off : C), 0,
                                                             R != nullptr ? span32 : 0, 0x00020000);   // no residual: reads give 0
@@ -427,8 +437,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int uni = ((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T);
-                        const short raw = __builtin_amdgcn_raw_buffer_load_b16(r_rsrc, lane_bytes, uni, 0);
-                        res[v] = Elem<T>::to_f32(__builtin_bit_cast(T, raw));
+                        if constexpr (sizeof(T) == 4) {
+                            res[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_rsrc, lane_bytes, uni, 0));
+                        } else {
+                            const short raw = __builtin_amdgcn_raw_buffer_load_b16(r_rsrc, lane_bytes, uni, 0);
+                            res[v] = Elem<T>::to_f32(__builtin_bit_cast(T, raw));
+                        }
                     }
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
@@ -440,7 +454,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     }
 }
 
-// fp32 path (parity configuration only; not a tuned kernel): 64x64 tile, 16-deep LDS slabs, 4x4 outputs
+// fp32 with ragged extents or unaligned tensors (not a tuned kernel): 64x64 tile, 16-deep LDS slabs, 4x4 outputs
 // per thread, plain FMA.
 template <int EPI>
 __global__ __launch_bounds__(256) void sgemm_nt_kernel(const float* __restrict__ A, const float* __restrict__ B0,
@@ -522,14 +536,27 @@ void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int
                        dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n, chip.xcds);
 }
 
+// k extent of one LDS stage of the DMA kernel: 128 bytes of a row for every element type
+template <typename T> constexpr int kStageK = 128 / (int)sizeof(T);
+
+// Ragged shapes: the bounds-checked kernels (register-staged MFMA for 16-bit, FMA for fp32).
+template <typename T, int EPI>
+void launch_ragged(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4)
+        hipLaunchKernelGGL((sgemm_nt_kernel<EPI>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, stream, A, B0, B1, C, R, M, N, K);
+    else
+        launch_gemm<T, 128, 128, EPI>(A, B0, B1, C, R, M, N, K, stream);
+}
+
 // Tile choice: 256-wide tiles (8 waves, two per SIMD) halve the L2 -> LDS traffic per MFMA but need one per CU to
 // occupy the chip; otherwise 128x128 tiles of 4 waves, which read a whole k-tile of fragments ahead (PF = 3): one
 // workgroup per CU with four stages in flight when every tile gets a CU of its own, two per CU with two stages else.
 template <typename T, int EPI>
 void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, int64_t tiles,
                         hipStream_t stream) {
-    if (tiles <= chip_info().cus) launch_gemm_dma<T, 128, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
-    else launch_gemm_dma<T, 128, 128, 2, 2, 64, 2, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+    constexpr int KT = kStageK<T>;
+    if (tiles <= chip_info().cus) launch_gemm_dma<T, 128, 128, 2, 2, KT, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+    else launch_gemm_dma<T, 128, 128, 2, 2, KT, 2, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
 }
 
 // Few tokens: 64-row tiles (wave tiles of 32 x 64 or 32 x 32), so that a batch of a few hundred tokens still gives
@@ -537,54 +564,41 @@ void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, 
 template <typename T, int EPI>
 void launch_narrow_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
     if (EPI == kEpiPlain && (int64_t)((M + 63) / 64) * (N / 128) < chip_info().cus && N % 64 == 0)
-        launch_gemm_dma<T, 64, 64, 2, 2, 64, 4, kEpiPlain, 3>(A, B0, B1, C, R, M, N, K, stream);
+        launch_gemm_dma<T, 64, 64, 2, 2, kStageK<T>, 4, kEpiPlain, 3>(A, B0, B1, C, R, M, N, K, stream);
     else
-        launch_gemm_dma<T, 64, 128, 2, 2, 64, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+        launch_gemm_dma<T, 64, 128, 2, 2, kStageK<T>, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
 }
 
 template <typename T>
-int gate_up_16bit(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
+int gate_up_tiled(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
     const T *A = (const T*)x, *G = (const T*)wg, *U = (const T*)wu, *S = (const T*)saved;
-    const bool k_ok = H % 64 == 0;
+    // the DMA kernel moves 16-byte pieces (fp32 callers need not align their tensors; those take the ragged kernel)
+    const bool k_ok = H % kStageK<T> == 0 && aligned16(x) && aligned16(wg) && aligned16(wu);
     if (k_ok && I % 128 == 0 && (int64_t)((M + 255) / 256) * (I / 128) >= chip_info().cus)
-        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, S, M, I, H, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, kStageK<T>, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, S, M, I, H, stream);
     else if (k_ok && I % 64 == 0 && (int64_t)((M + 127) / 128) * (I / 64) >= chip_info().cus)
         launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, (int64_t)((M + 127) / 128) * (I / 64), stream);
     else if (k_ok && I % 64 == 0)
         launch_narrow_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
     else
-        launch_gemm<T, 128, 128, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
+        launch_ragged<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up)");
     return FMOE_OK;
 }
 
 template <typename T>
-int down_16bit(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
+int down_tiled(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
     const T *A = (const T*)h, *W = (const T*)wd, *R = (const T*)residual;
-    const bool k_ok = I % 64 == 0;
+    const bool k_ok = I % kStageK<T> == 0 && aligned16(h) && aligned16(wd);
     if (k_ok && H % 256 == 0 && (int64_t)((M + 255) / 256) * (H / 256) >= chip_info().cus)
-        launch_gemm_dma<T, 256, 256, 2, 4, 64, 2, kEpiPlain, 1>(A, W, nullptr, (T*)out, R, M, H, I, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, kStageK<T>, 2, kEpiPlain, 1>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     else if (k_ok && H % 128 == 0 && (int64_t)((M + 127) / 128) * (H / 128) >= chip_info().cus)
         launch_small_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, (int64_t)((M + 127) / 128) * (H / 128), stream);
     else if (k_ok && H % 128 == 0)
         launch_narrow_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     else
-        launch_gemm<T, 128, 128, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
+        launch_ragged<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     FMOE_CHECK_LAUNCH("fmoe_mlp(down)");
-    return FMOE_OK;
-}
-
-int gate_up_f32(const void* x, const void* wg, const void* wu, int M, int H, int I, void* h, void* saved, hipStream_t stream) {
-    hipLaunchKernelGGL((sgemm_nt_kernel<kEpiSwiGLU>), dim3((I + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
-                       (const float*)x, (const float*)wg, (const float*)wu, (float*)h, (const float*)saved, M, I, H);
-    FMOE_CHECK_LAUNCH("fmoe_mlp(gate/up, f32)");
-    return FMOE_OK;
-}
-
-int down_f32(const void* h, const void* wd, int M, int H, int I, const void* residual, void* out, hipStream_t stream) {
-    hipLaunchKernelGGL((sgemm_nt_kernel<kEpiPlain>), dim3((H + 63) / 64, (M + 63) / 64), dim3(256), 0, stream,
-                       (const float*)h, (const float*)wd, nullptr, (float*)out, (const float*)residual, M, H, I);
-    FMOE_CHECK_LAUNCH("fmoe_mlp(down, f32)");
     return FMOE_OK;
 }
 
@@ -620,9 +634,9 @@ int mlp_gate_up_impl(const char* who, const void* x, const void* gate_w, const v
     hipStream_t s = (hipStream_t)stream;
     const int M = (int)num_tokens;
     switch (dtype) {
-        case FMOE_F32: return gate_up_f32(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
-        case FMOE_BF16: return gate_up_16bit<bf16_t>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
-        default: return gate_up_16bit<f16_t>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
+        case FMOE_F32: return gate_up_tiled<float>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
+        case FMOE_BF16: return gate_up_tiled<bf16_t>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
+        default: return gate_up_tiled<f16_t>(x, gate_w, up_w, M, hidden, intermediate, act, saved, s);
     }
 }
 }  // namespace
@@ -656,9 +670,9 @@ extern "C" int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_to
     hipStream_t s = (hipStream_t)stream;
     const int M = (int)num_tokens;
     switch (dtype) {
-        case FMOE_F32: return down_f32(act, down_w, M, hidden, intermediate, residual, out, s);
-        case FMOE_BF16: return down_16bit<bf16_t>(act, down_w, M, hidden, intermediate, residual, out, s);
-        default: return down_16bit<f16_t>(act, down_w, M, hidden, intermediate, residual, out, s);
+        case FMOE_F32: return down_tiled<float>(act, down_w, M, hidden, intermediate, residual, out, s);
+        case FMOE_BF16: return down_tiled<bf16_t>(act, down_w, M, hidden, intermediate, residual, out, s);
+        default: return down_tiled<f16_t>(act, down_w, M, hidden, intermediate, residual, out, s);
     }
 }
 

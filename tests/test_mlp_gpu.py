@@ -35,8 +35,6 @@ def truth64(x, wg, wu, wd):
 def test_mlp_matches_oracle(dtype, T, H, I):
     from flash_moe.ops import flash_mlp_func
 
-    if dtype == torch.float32 and T * H * I > 1024 * 1024 * 4096:
-        pytest.skip("fp32 is the small parity configuration only")
     x, wg, wu, wd = make(T, H, I, dtype, seed=T + I)
     got = flash_mlp_func(*cuda(x, wg, wu, wd)).cpu()
     assert got.dtype == dtype and got.shape == (T, H)
@@ -45,6 +43,26 @@ def test_mlp_matches_oracle(dtype, T, H, I):
     assert rel_fro(got, ref64) < {torch.float32: 2e-6, torch.bfloat16: 6e-3, torch.float16: 8e-4}[dtype]
     if T <= 1024:
         assert_output_close(got, orc.mlp_forward(x, wg, wu, wd), dtype, "mlp vs same-dtype oracle")
+
+
+def test_mlp_fp32_tensors_off_the_16_byte_grid():
+    # fp32 callers need not align their tensors: the tiled kernel moves 16-byte pieces, so these take the bounds-checked
+    # kernel, and the result is the aligned one's up to summation order
+    from flash_moe.ops import flash_mlp_func
+
+    x, wg, wu, wd = cuda(*make(256, 256, 512, torch.float32, seed=9))
+
+    def shifted(t):
+        buf = torch.empty(t.numel() + 1, device="cuda", dtype=t.dtype)
+        buf[1:].copy_(t.reshape(-1))
+        v = buf[1:].view(t.shape)
+        assert v.data_ptr() % 16 == 4
+        return v
+
+    aligned = flash_mlp_func(x, wg, wu, wd)
+    moved = flash_mlp_func(shifted(x), shifted(wg), shifted(wu), shifted(wd))
+    ref64 = truth64(*(t.cpu() for t in (x, wg, wu, wd)))
+    assert rel_fro(aligned, ref64) < 2e-6 and rel_fro(moved, ref64) < 2e-6
 
 
 def test_mlp_reference_test_distribution():
