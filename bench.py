@@ -209,6 +209,11 @@ def roofline_entry(name, ms, w, traffic, launches=None, spread_us=None):
     if spread_us is not None:
         entry["median_launch_us"], entry["min_launch_us"], entry["max_launch_us"] = (spread_us["median"], spread_us["min"],
                                                                                       spread_us["max"])
+    clock = measured_traffic(name, "clock_ghz_c4")
+    if clock is not None:
+        # shader clock while this kernel runs, from the kept counter summary (profiles/mlp_c4_counters.txt): the peak above
+        # is quoted at 2.4 GHz
+        entry["clock_ghz"] = clock
     if w["bound"] == "hbm" and "flops" in w:
         # a contraction below the MFMA ridge: the matrix-core fraction next to the binding (HBM) one
         tf = w["flops"] / (ms * 1e-3) / 1e12
@@ -584,7 +589,7 @@ def main():
         result["block_c5"] = bench_block_c5(dtype, 5)
         log("block C5:", result["block_c5"])
         torch.cuda.empty_cache()
-        result["mlp_fp32"] = bench_mlp_fp32(10)
+        result["mlp_fp32"] = result["rooflines_all"]["mlp_fp32"] = bench_mlp_fp32(10)
         log("mlp fp32:", result["mlp_fp32"])
         result["backward_c4"] = bench_backward_c4(dtype, 10)
         log("backward C4:", result["backward_c4"])

@@ -59,7 +59,11 @@ const char* fmoe_last_error(void);
  *   scores     [num_tokens, top_k]        dtype      K largest sums lp[0,t,i]+lp[1,t,j], descending;
  *                                                    16-bit dtypes: each sum rounded to dtype, as the
  *                                                    reference adds in the input dtype (flash_router.py:51-53)
- *   indices    [num_tokens, top_k]        int64      i*num_keys + j; ties to the lower index (tl.argmax rule)
+ *   indices    [num_tokens, top_k]        int64      i*num_keys + j.  Equal sums at the cut: with num_keys <= 512 and
+ *                                                    top_k <= 128 (the register-resident selection) the entries equal to
+ *                                                    the K-th sum are taken in candidate order (rank in half 0, then
+ *                                                    rank in half 1); otherwise the lower flat index wins (tl.argmax
+ *                                                    rule).  The scores are the same either way.
  *   gates      [num_tokens, top_k]        dtype      optional (NULL to skip): exp(score), divided by the
  *                                                    per-token sum when norm_topk_prob != 0
  * Requires 0 <= top_k <= num_keys (same rule as the reference's assert).
