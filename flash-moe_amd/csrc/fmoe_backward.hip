@@ -30,42 +30,54 @@ template <typename T>
 __global__ __launch_bounds__(kBwdWaves* kWave) void router_backward_kernel(const T* __restrict__ dscores,
                                                                            const int64_t* __restrict__ indices,
                                                                            T* __restrict__ dlogits, int64_t num_tokens,
-                                                                           int nk, int top_k, int waves_per_block) {
-    extern __shared__ float acc_all[];   // [waves_per_block][2 * nk], one private row pair per wave
+                                                                           int nk, int top_k, int waves_per_block, int chunk) {
+    extern __shared__ float acc_all[];   // [waves_per_block][2 * chunk], one private row pair per wave
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
     const int64_t token = (int64_t)blockIdx.x * waves_per_block + wave;
     if (wave >= waves_per_block || token >= num_tokens) return;   // whole waves leave; nobody waits on them
-    float* acc = acc_all + (size_t)wave * 2 * nk;
-    for (int p = lane; p < 2 * nk; p += kWave) acc[p] = 0.0f;
-    __builtin_amdgcn_wave_barrier();
+    float* acc = acc_all + (size_t)wave * 2 * chunk;
     const int64_t num_pairs = (int64_t)nk * nk;
-    // LDS adds of one instruction that hit the same address are applied one after the other by the LDS unit, and the
-    // instructions of a wave execute in order, so the sum has a fixed order for given inputs
-    for (int k = lane; k < top_k; k += kWave) {
-        const int64_t id = indices[token * top_k + k];
-        if (id >= 0 && id < num_pairs) {
-            const float d = Elem<T>::to_f32(dscores[token * top_k + k]);
-            __hip_atomic_fetch_add(&acc[(int)(id / nk)], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-            __hip_atomic_fetch_add(&acc[nk + (int)(id % nk)], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    // The two gradient rows are built `chunk` keys at a time (chunk = nk when a row pair fits the LDS): per chunk the
+    // pairs are scanned again and only the keys inside it are added.
+    for (int c0 = 0; c0 < nk; c0 += chunk) {
+        const int cn = nk - c0 < chunk ? nk - c0 : chunk;
+        for (int p = lane; p < 2 * chunk; p += kWave) acc[p] = 0.0f;
+        __builtin_amdgcn_wave_barrier();
+        // LDS adds of one instruction that hit the same address are applied one after the other by the LDS unit, and the
+        // instructions of a wave execute in order, so the sum has a fixed order for given inputs
+        for (int k = lane; k < top_k; k += kWave) {
+            const int64_t id = indices[token * top_k + k];
+            if (id >= 0 && id < num_pairs) {
+                const float d = Elem<T>::to_f32(dscores[token * top_k + k]);
+                const int i = (int)(id / nk) - c0, j = (int)(id % nk) - c0;
+                if (i >= 0 && i < cn) __hip_atomic_fetch_add(&acc[i], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                if (j >= 0 && j < cn) __hip_atomic_fetch_add(&acc[chunk + j], d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            }
         }
-    }
-    __builtin_amdgcn_wave_barrier();
-    for (int p = lane; p < nk; p += kWave) {
-        dlogits[token * nk + p] = Elem<T>::from_f32(acc[p]);
-        dlogits[(num_tokens + token) * nk + p] = Elem<T>::from_f32(acc[nk + p]);
+        __builtin_amdgcn_wave_barrier();
+        for (int p = lane; p < cn; p += kWave) {
+            dlogits[token * nk + c0 + p] = Elem<T>::from_f32(acc[p]);
+            dlogits[(num_tokens + token) * nk + c0 + p] = Elem<T>::from_f32(acc[chunk + p]);
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
+
+// Keys of a half whose gradient row is held in LDS at a time: the whole half up to 8192 keys (64 KiB for the pair of
+// rows), 4096 beyond.
+inline int backward_key_chunk(int nk) { return nk <= 8192 ? nk : 4096; }
 
 template <typename T>
 int launch_router_backward(const void* dscores, const int64_t* indices, void* dlogits, int64_t T_, int nk, int K,
                            hipStream_t stream) {
-    const size_t per_wave = (size_t)2 * nk * sizeof(float);
+    const int chunk = backward_key_chunk(nk);
+    const size_t per_wave = (size_t)2 * chunk * sizeof(float);
     int waves = (int)((48 * 1024) / per_wave);
     waves = waves < 1 ? 1 : (waves > kBwdWaves ? kBwdWaves : waves);
     const unsigned grid = (unsigned)((T_ + waves - 1) / waves);
     hipLaunchKernelGGL((router_backward_kernel<T>), dim3(grid), dim3(kBwdWaves * kWave), waves * per_wave, stream,
-                       (const T*)dscores, indices, (T*)dlogits, T_, nk, K, waves);
+                       (const T*)dscores, indices, (T*)dlogits, T_, nk, K, waves, chunk);
     FMOE_CHECK_LAUNCH("fmoe_router_topk_backward");
     return FMOE_OK;
 }
@@ -82,13 +94,13 @@ template <typename T>
 __global__ __launch_bounds__(kBwdWaves* kWave) void route_backward_kernel(
     const T* __restrict__ dgates, const int64_t* __restrict__ indices, const float* __restrict__ logits,
     const T* __restrict__ dlogits_extra, float* __restrict__ dlogits, int64_t num_tokens, int nk, int top_k,
-    int norm_topk_prob, int waves_per_block) {
-    extern __shared__ float acc_all[];   // [waves_per_block][2 * nk], one private row pair per wave
+    int norm_topk_prob, int waves_per_block, int chunk) {
+    extern __shared__ float acc_all[];   // [waves_per_block][2 * chunk], one private row pair per wave
     const int lane = lane_id();
     const int wave = (int)(threadIdx.x >> 6);
     const int64_t token = (int64_t)blockIdx.x * waves_per_block + wave;
     if (wave >= waves_per_block || token >= num_tokens) return;   // whole waves leave; nobody waits on them
-    float* acc = acc_all + (size_t)wave * 2 * nk;
+    float* acc = acc_all + (size_t)wave * 2 * chunk;
     const float* row = logits + token * 2 * nk;
     float shift[2], lse[2];
 #pragma unroll
@@ -101,8 +113,6 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void route_backward_kernel(
         shift[h] = mx;
         lse[h] = logf(wave_sum(se));
     }
-    for (int p = lane; p < 2 * nk; p += kWave) acc[p] = 0.0f;
-    __builtin_amdgcn_wave_barrier();
     const int64_t num_pairs = (int64_t)nk * nk;
     // first pass (renormalised gates only): sum_m e_m and sum_m dg_m e_m
     float total = 1.0f, dot = 0.0f;
@@ -120,43 +130,71 @@ __global__ __launch_bounds__(kBwdWaves* kWave) void route_backward_kernel(
         total = wave_sum(te);
         dot = wave_sum(td) / total;          // sum_m dg_m g_m
     }
-    // LDS adds of one instruction that hit the same address are applied one after the other by the LDS unit, and the
-    // instructions of a wave execute in order, so the sum has a fixed order for given inputs
-    for (int k = lane; k < top_k; k += kWave) {
-        const int64_t id = indices[token * top_k + k];
-        if (id >= 0 && id < num_pairs) {
-            const int i = (int)(id / nk), j = (int)(id % nk);
-            const float e = expf(((row[i] - shift[0]) - lse[0]) + ((row[nk + j] - shift[1]) - lse[1]));
-            const float dg = Elem<T>::to_f32(dgates[token * top_k + k]);
-            const float ds = norm_topk_prob ? (e / total) * (dg - dot) : dg * e;
-            __hip_atomic_fetch_add(&acc[i], ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-            __hip_atomic_fetch_add(&acc[nk + j], ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    // The two gradient rows are built `chunk` keys at a time (chunk = nk when a row pair fits the LDS): per chunk the
+    // pairs are scanned again and only the keys inside it are added.  With several chunks the row totals, which every
+    // key's result needs, are the sum of the pair gradients themselves (each valid pair adds to one key of either half).
+    const bool chunked = chunk < nk;
+    float sum_all = 0.0f;
+    if (chunked) {
+        float part = 0.0f;
+        for (int k = lane; k < top_k; k += kWave) {
+            const int64_t id = indices[token * top_k + k];
+            if (id >= 0 && id < num_pairs) {
+                const int i = (int)(id / nk), j = (int)(id % nk);
+                const float e = expf(((row[i] - shift[0]) - lse[0]) + ((row[nk + j] - shift[1]) - lse[1]));
+                const float dg = Elem<T>::to_f32(dgates[token * top_k + k]);
+                part += norm_topk_prob ? (e / total) * (dg - dot) : dg * e;
+            }
         }
+        sum_all = wave_sum(part);
     }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        float sum = 0.0f;
-        for (int p = lane; p < nk; p += kWave) sum += acc[h * nk + p];
-        sum = wave_sum(sum);
-        for (int p = lane; p < nk; p += kWave) {
-            const int64_t at = token * 2 * nk + h * nk + p;
-            float d = acc[h * nk + p] - expf((row[h * nk + p] - shift[h]) - lse[h]) * sum;
-            if (dlogits_extra != nullptr) d += Elem<T>::to_f32(dlogits_extra[at]);
-            dlogits[at] = d;
+    for (int c0 = 0; c0 < nk; c0 += chunk) {
+        const int cn = nk - c0 < chunk ? nk - c0 : chunk;
+        for (int p = lane; p < 2 * chunk; p += kWave) acc[p] = 0.0f;
+        __builtin_amdgcn_wave_barrier();
+        // LDS adds of one instruction that hit the same address are applied one after the other by the LDS unit, and the
+        // instructions of a wave execute in order, so the sum has a fixed order for given inputs
+        for (int k = lane; k < top_k; k += kWave) {
+            const int64_t id = indices[token * top_k + k];
+            if (id >= 0 && id < num_pairs) {
+                const int i = (int)(id / nk), j = (int)(id % nk);
+                const float e = expf(((row[i] - shift[0]) - lse[0]) + ((row[nk + j] - shift[1]) - lse[1]));
+                const float dg = Elem<T>::to_f32(dgates[token * top_k + k]);
+                const float ds = norm_topk_prob ? (e / total) * (dg - dot) : dg * e;
+                if (i >= c0 && i < c0 + cn) __hip_atomic_fetch_add(&acc[i - c0], ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                if (j >= c0 && j < c0 + cn) __hip_atomic_fetch_add(&acc[chunk + j - c0], ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            }
         }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float sum = sum_all;
+            if (!chunked) {
+                sum = 0.0f;
+                for (int p = lane; p < nk; p += kWave) sum += acc[h * chunk + p];
+                sum = wave_sum(sum);
+            }
+            for (int p = lane; p < cn; p += kWave) {
+                const int64_t at = token * 2 * nk + h * nk + c0 + p;
+                float d = acc[h * chunk + p] - expf((row[h * nk + c0 + p] - shift[h]) - lse[h]) * sum;
+                if (dlogits_extra != nullptr) d += Elem<T>::to_f32(dlogits_extra[at]);
+                dlogits[at] = d;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
 template <typename T>
 int launch_route_backward(const void* dgates, const int64_t* indices, const float* logits, const void* dlogits_extra,
                           float* dlogits, int64_t T_, int nk, int K, int norm, hipStream_t stream) {
-    const size_t per_wave = (size_t)2 * nk * sizeof(float);
+    const int chunk = backward_key_chunk(nk);
+    const size_t per_wave = (size_t)2 * chunk * sizeof(float);
     int waves = (int)((48 * 1024) / per_wave);
     waves = waves < 1 ? 1 : (waves > kBwdWaves ? kBwdWaves : waves);
     const unsigned grid = (unsigned)((T_ + waves - 1) / waves);
     hipLaunchKernelGGL((route_backward_kernel<T>), dim3(grid), dim3(kBwdWaves * kWave), waves * per_wave, stream,
-                       (const T*)dgates, indices, logits, (const T*)dlogits_extra, dlogits, T_, nk, K, norm, waves);
+                       (const T*)dgates, indices, logits, (const T*)dlogits_extra, dlogits, T_, nk, K, norm, waves, chunk);
     FMOE_CHECK_LAUNCH("fmoe_route_backward");
     return FMOE_OK;
 }
@@ -526,7 +564,7 @@ extern "C" int fmoe_router_topk_backward(const void* dscores, const int64_t* ind
     FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_router_topk_backward: unknown dtype %d", dtype);
     FMOE_REQUIRE(num_tokens >= 0 && num_keys > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
                  "fmoe_router_topk_backward: bad shape T=%lld nk=%d K=%d", (long long)num_tokens, num_keys, top_k);
-    FMOE_REQUIRE(num_keys <= 8192, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk_backward: num_keys=%d > 8192", num_keys);
+    FMOE_REQUIRE(num_keys <= 65535, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk_backward: num_keys=%d > 65535", num_keys);
     if (num_tokens == 0) return FMOE_OK;
     FMOE_REQUIRE(drouter_logits && (top_k == 0 || (dscores && indices)), FMOE_ERR_NULL_POINTER,
                  "fmoe_router_topk_backward: null tensor pointer");
@@ -546,7 +584,7 @@ extern "C" int fmoe_route_backward(const void* dgates, const int64_t* indices, c
     FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "fmoe_route_backward: unknown dtype %d", dtype);
     FMOE_REQUIRE(num_tokens >= 0 && num_keys > 0 && top_k >= 0, FMOE_ERR_BAD_SHAPE,
                  "fmoe_route_backward: bad shape T=%lld nk=%d K=%d", (long long)num_tokens, num_keys, top_k);
-    FMOE_REQUIRE(num_keys <= 8192, FMOE_ERR_UNSUPPORTED, "fmoe_route_backward: num_keys=%d > 8192", num_keys);
+    FMOE_REQUIRE(num_keys <= 32767, FMOE_ERR_UNSUPPORTED, "fmoe_route_backward: num_keys=%d > 32767", num_keys);
     if (num_tokens == 0) return FMOE_OK;
     FMOE_REQUIRE(logits_fp32 && dlogits_fp32 && (top_k == 0 || (dgates && indices)), FMOE_ERR_NULL_POINTER,
                  "fmoe_route_backward: null tensor pointer");

@@ -26,7 +26,6 @@ the module dtype as in the reference.
 from __future__ import annotations
 
 import math
-import warnings
 
 import torch
 import torch.nn as nn
@@ -38,7 +37,6 @@ from flash_moe.ops.hip.flash_mlp import flash_mlp_func, mlp_forward
 from flash_moe.ops.hip.flash_router import flash_router_func, router_forward, router_prologue
 
 _SILU_NAMES = ("silu", "swish")
-BACKWARD_MAX_NUM_KEYS = 8192     # limit of the routing stage's backward entry points (the forward's is 32767)
 
 
 class FlashMoEConfig:
@@ -69,12 +67,6 @@ class FlashMoE(nn.Module):
         self.act_fn = F.silu
         # experts are addressed by a pair of sub-keys; ids >= num_keys**2 are never selected (:38)
         self.num_keys = math.floor(math.sqrt(E))
-        if self.num_keys > BACKWARD_MAX_NUM_KEYS:
-            # the forward routes up to 32767 sub-keys per half; fmoe_route_backward / fmoe_router_topk_backward keep a
-            # token's two gradient rows in LDS and stop at 8192
-            warnings.warn(f"num_experts={E} gives {self.num_keys} sub-keys per half: the forward runs, but the backward "
-                          f"pass of the routing stage supports at most {BACKWARD_MAX_NUM_KEYS} and will raise",
-                          RuntimeWarning, stacklevel=2)
         self.top_k = config.num_experts_per_tok
         self.norm_topk_prob = config.norm_topk_prob
 

@@ -286,7 +286,7 @@ int fmoe_pkm_forward(const void* values, const void* routing_weights, const int6
  * 205-249): drouter_logits [2, T, nk] (dtype), fully written:
  *   [0,t,i] = sum of dscores[t,k] over k with indices[t,k] / nk == i;  [1,t,j] likewise with indices[t,k] % nk.
  * dscores [T, K] dtype, indices [T, K] int64 (ids outside [0, nk*nk) contribute nothing).
- * Limit of this build: num_keys <= 8192 (the forward routes up to 32767). */
+ * Limit of this build: num_keys <= 65535, as fmoe_router_topk. */
 int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64_t num_tokens, int num_keys, int top_k,
                               int dtype, void* drouter_logits, void* stream);
 
@@ -297,7 +297,7 @@ int fmoe_router_topk_backward(const void* dscores, const int64_t* indices, int64
  *   [0, nk*nk) contribute nothing); logits_fp32 [T, 2*nk]: the fp32 gate logits the forward routed from
  *   (router_logits_fp32 of fmoe_router_forward); dlogits_extra [T, 2*nk] dtype or NULL: gradient of the returned
  *   router logits, added to the result; dlogits_fp32 [T, 2*nk] fp32, fully written: what
- *   fmoe_router_prologue_backward takes.  Limit of this build: num_keys <= 8192. */
+ *   fmoe_router_prologue_backward takes.  Limit of this build: num_keys <= 32767, as fmoe_router_forward. */
 int fmoe_route_backward(const void* dgates, const int64_t* indices, const float* logits_fp32, const void* dlogits_extra,
                         int64_t num_tokens, int num_keys, int top_k, int dtype, int norm_topk_prob, float* dlogits_fp32,
                         void* stream);

@@ -172,13 +172,13 @@ def test_backward_argument_checks():
     rb = lib.fmoe_router_topk_backward
     assert rb(a, a, 4, 8, 2, 9, a, None) == -4
     assert rb(a, a, 4, 0, 2, _C.F32, a, None) == -2
-    assert rb(a, a, 4, 9000, 2, _C.F32, a, None) == -5
+    assert rb(a, a, 4, 70000, 2, _C.F32, a, None) == -5                          # the forward op's own key limit
     assert rb(a, None, 4, 8, 2, _C.F32, a, None) == -1
     assert rb(None, None, 0, 8, 2, _C.F32, None, None) == 0
     rt = lib.fmoe_route_backward
     assert rt(a, a, a, None, 4, 8, 2, 9, 0, a, None) == -4                       # dtype
     assert rt(a, a, a, None, 4, 0, 2, _C.BF16, 0, a, None) == -2                 # num_keys
-    assert rt(a, a, a, None, 4, 9000, 2, _C.BF16, 0, a, None) == -5              # more keys than the LDS rows hold
+    assert rt(a, a, a, None, 4, 40000, 2, _C.BF16, 0, a, None) == -5             # the fused router's own key limit
     assert rt(a, a, None, None, 4, 8, 2, _C.BF16, 0, a, None) == -1              # logits
     assert rt(None, None, a, None, 4, 8, 2, _C.BF16, 0, a, None) == -1           # gate gradient with top_k > 0
     assert rt(None, None, None, None, 0, 8, 2, _C.BF16, 1, None, None) == 0      # empty batch

@@ -16,7 +16,8 @@ def gen(seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("T,nk,K", [(64, 32, 16), (300, 128, 64), (17, 512, 128), (5, 8, 1)])
+@pytest.mark.parametrize("T,nk,K", [(64, 32, 16), (300, 128, 64), (17, 512, 128), (5, 8, 1),
+                                    (6, 9000, 48)])    # more keys than one LDS row pair holds: rows built 4096 keys at a time
 def test_router_backward(dtype, T, nk, K):
     from flash_moe.ops import flash_router_func
     from flash_moe.ops.hip.flash_router import router_topk_backward
@@ -45,14 +46,19 @@ def test_router_backward(dtype, T, nk, K):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("norm", [False, True])
-@pytest.mark.parametrize("T,nk,K", [(64, 32, 16), (130, 128, 64), (9, 512, 128), (5, 8, 1)])
+@pytest.mark.parametrize("T,nk,K", [(64, 32, 16), (130, 128, 64), (9, 512, 128), (5, 8, 1),
+                                    (5, 8192, 64), (6, 20000, 96)])   # the last: rows built 4096 keys at a time
 def test_route_backward(dtype, norm, T, nk, K):
     """Gate gradients -> gradient of the fp32 gate logits, against float64 autograd of log-softmax, pair sums, exp and
     renormalisation on the same ids; ids out of range carry nothing; the gradient of the returned logits is added."""
     from flash_moe.ops.hip.flash_router import route_backward
 
     logits = torch.randn(T, 2 * nk, generator=gen(1)) * 2.0
-    idx = torch.stack([torch.randperm(nk * nk, generator=gen(10 + t))[:K] for t in range(T)])
+    if nk <= 512:
+        idx = torch.stack([torch.randperm(nk * nk, generator=gen(10 + t))[:K] for t in range(T)])
+    else:   # pairs that share keys (several gradients per key) and lie on both sides of every 4096-key boundary
+        idx = torch.randint(0, nk, (T, K), generator=gen(10)) * nk + torch.randint(0, nk, (T, K), generator=gen(11))
+        idx[:, : K // 2] = idx[:, K // 2 : 2 * (K // 2)] // nk * nk + (idx[:, : K // 2] % nk)
     if K > 2:
         idx[::3, 1] = nk * nk + 7
         idx[1::4, 2] = -1

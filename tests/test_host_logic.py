@@ -37,19 +37,6 @@ def test_module_rejects_other_activations():
         FlashMoE(FlashMoEConfig(64, 128, "gelu", 100, 4))
 
 
-def test_module_warns_beyond_the_routing_backward_limit():
-    # the forward routes up to 32767 sub-keys per half, the routing backward 8192: a module beyond that says so at construction
-    import warnings
-
-    with torch.device("meta"):
-        with pytest.warns(RuntimeWarning, match="backward"):
-            m = FlashMoE(FlashMoEConfig(8, 16, "silu", 8193 * 8193, 4))
-        assert m.num_keys == 8193
-        with warnings.catch_warnings():
-            warnings.simplefilter("error")
-            FlashMoE(FlashMoEConfig(8, 16, "silu", 1024, 4))
-
-
 def test_forward_signature():
     sig = inspect.signature(FlashMoE.forward)
     assert list(sig.parameters)[:2] == ["self", "hidden_states"]
