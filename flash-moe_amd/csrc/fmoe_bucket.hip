@@ -206,6 +206,174 @@ __global__ __launch_bounds__(kOrderWaves* kWave) void bucket_order_kernel(
     }
 }
 
+// ---- grouping by two partition passes --------------------------------------------------------------------------------
+// For millions of pairs the histogram and the fill above are bound by the rate of global atomics (20-28 G/s) and by
+// scattered 4-byte writes.  Here no global atomic is issued: the pairs are first partitioned into at most 1024 coarse
+// buckets of 2^shift consecutive experts (per tile of pairs a histogram in LDS, one scan over (bucket, tile), then each tile
+// writes its pairs behind its own offsets), and one workgroup per coarse bucket finishes it in LDS (counts per expert,
+// scan = the expert offsets, slots handed out by LDS cursors).  Pairs with an id outside [0, E) form one more bucket at the
+// end, whose slots are the zeroed tail.  The order inside an expert's segment is whatever the LDS serves first.
+// pairs per workgroup of the partition passes: long runs per (tile, bucket) for millions of pairs, more workgroups for fewer
+inline int partition_tile(int64_t num_pairs) { return num_pairs >= (1ll << 21) ? 8192 : 2048; }
+constexpr int kPartMaxBuckets = 1024;    // coarse buckets, not counting the one for invalid ids
+constexpr int kPartMaxShift = 13;        // 2^13 experts per coarse bucket: 32 KiB of LDS counters
+
+__global__ __launch_bounds__(256) void partition_count_kernel(const int64_t* __restrict__ indices, int32_t* __restrict__ counts1,
+                                                              int64_t num_pairs, int64_t num_experts, int shift, int buckets,
+                                                              int groups, int tile, int32_t* __restrict__ ticket,
+                                                              uint64_t* __restrict__ status, int tiles) {
+    __shared__ int32_t hist[kPartMaxBuckets + 1];
+    const int g = (int)blockIdx.x, tid = (int)threadIdx.x;
+    if (g == 0) {      // the state of the scan that follows
+        if (tid == 0) *ticket = 0;
+        for (int i = tid; i < tiles; i += 256) status[i] = 0;
+    }
+    for (int b = tid; b <= buckets; b += 256) hist[b] = 0;
+    __syncthreads();
+    const int64_t p0 = (int64_t)g * tile;
+    for (int i = tid; i < tile; i += 256) {
+        const int64_t p = p0 + i;
+        if (p < num_pairs) {
+            const int64_t e = indices[p];
+            atomicAdd(&hist[(e >= 0 && e < num_experts) ? (int)(e >> shift) : buckets], 1);
+        }
+    }
+    __syncthreads();
+    for (int b = tid; b <= buckets; b += 256) counts1[(int64_t)b * groups + g] = hist[b];
+}
+
+// stage[slot] = pair index << 32 | id inside its coarse bucket (all ones for an invalid id)
+__global__ __launch_bounds__(256) void partition_scatter_kernel(const int64_t* __restrict__ indices,
+                                                                const int32_t* __restrict__ offs1, uint64_t* __restrict__ stage,
+                                                                float* __restrict__ coef_clear, int64_t num_pairs,
+                                                                int64_t num_experts, int shift, int buckets, int groups,
+                                                                int tile) {
+    __shared__ int32_t base[kPartMaxBuckets + 1];
+    const int g = (int)blockIdx.x, tid = (int)threadIdx.x;
+    for (int b = tid; b <= buckets; b += 256) base[b] = offs1[(int64_t)b * groups + g];
+    __syncthreads();
+    const int64_t p0 = (int64_t)g * tile;
+    for (int i = tid; i < tile; i += 256) {
+        const int64_t p = p0 + i;
+        if (p < num_pairs) {
+            const int64_t e = indices[p];
+            const bool ok = e >= 0 && e < num_experts;
+            const int b = ok ? (int)(e >> shift) : buckets;
+            const int32_t slot = atomicAdd(&base[b], 1);
+            stage[slot] = ((uint64_t)(uint32_t)p << 32) | (ok ? (uint32_t)(e - ((int64_t)b << shift)) : 0xFFFFFFFFu);
+            if (!ok && coef_clear != nullptr) coef_clear[p] = 0.0f;
+        }
+    }
+}
+
+constexpr int kPartLocalThreads = 512;
+constexpr int kPartLocalCap = 8192;      // pairs of a coarse bucket that are put in order in LDS and written out coalesced
+
+__global__ __launch_bounds__(kPartLocalThreads) void partition_local_kernel(
+    const uint64_t* __restrict__ stage, const int32_t* __restrict__ offs1, int32_t* __restrict__ offsets,
+    int32_t* __restrict__ sorted_pairs, uint32_t* __restrict__ tok, uint32_t* __restrict__ exp, int64_t num_experts, int shift,
+    int buckets, int groups, int top_k, uint32_t tok_scale, uint32_t exp_scale, int pack_shift) {
+    extern __shared__ int32_t cnt[];     // 1 << shift
+    __shared__ uint32_t out_pair[kPartLocalCap];
+    __shared__ uint16_t out_low[kPartLocalCap];
+    __shared__ int32_t wave_total[kPartLocalThreads / kWave];
+    constexpr int NT = kPartLocalThreads;
+    const int b = (int)blockIdx.x, tid = (int)threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+    const int32_t begin = offs1[(int64_t)b * groups], end = offs1[(int64_t)(b + 1) * groups];
+    if (b == buckets) {      // the slots after the last segment
+        if (tid == 0) offsets[num_experts] = begin;
+        for (int32_t s = begin + tid; s < end; s += NT) {
+            if (tok != nullptr) tok[s] = 0u;
+            if (exp != nullptr) exp[s] = 0u;
+        }
+        return;
+    }
+    const int64_t e0 = (int64_t)b << shift;
+    const int n_e = (int)(num_experts - e0 < (1ll << shift) ? num_experts - e0 : (1ll << shift));
+    for (int j = tid; j < n_e; j += NT) cnt[j] = 0;
+    __syncthreads();
+    for (int32_t s = begin + tid; s < end; s += 2 * NT) {
+        const uint64_t v0 = stage[s], v1 = s + NT < end ? stage[s + NT] : 0;
+        atomicAdd(&cnt[(uint32_t)v0], 1);
+        if (s + NT < end) atomicAdd(&cnt[(uint32_t)v1], 1);
+    }
+    __syncthreads();
+    // exclusive scan of the counts: thread t owns experts [t * per, (t + 1) * per)
+    const int per = (n_e + NT - 1) / NT;
+    const int j0 = tid * per < n_e ? tid * per : n_e, j1 = j0 + per < n_e ? j0 + per : n_e;
+    int32_t mine = 0;
+    for (int j = j0; j < j1; ++j) mine += cnt[j];
+    int32_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_total[wave] = incl;
+    __syncthreads();
+    int32_t run = begin + incl - mine;
+    for (int w = 0; w < wave; ++w) run += wave_total[w];
+    for (int j = j0; j < j1; ++j) {
+        const int32_t c = cnt[j];
+        offsets[e0 + j] = run;
+        cnt[j] = run;            // the cursor of expert e0 + j
+        run += c;
+    }
+    __syncthreads();
+    auto emit = [&](int32_t slot, uint32_t p, uint32_t low) {
+        const uint32_t e = (uint32_t)e0 + low;
+        sorted_pairs[slot] = (int32_t)p;
+        if (tok != nullptr) tok[slot] = (p / (uint32_t)top_k) * tok_scale | (pack_shift ? e << pack_shift : 0u);
+        if (exp != nullptr) exp[slot] = e * exp_scale;
+    };
+    const bool in_lds = end - begin <= kPartLocalCap;      // else (a few experts took a large share of all pairs): slot by slot
+    for (int32_t s = begin + tid; s < end; s += 2 * NT) {
+        const bool two = s + NT < end;
+        const uint64_t v0 = stage[s], v1 = two ? stage[s + NT] : 0;
+        const int32_t slot0 = atomicAdd(&cnt[(uint32_t)v0], 1);
+        const int32_t slot1 = two ? atomicAdd(&cnt[(uint32_t)v1], 1) : 0;
+        if (in_lds) {
+            out_pair[slot0 - begin] = (uint32_t)(v0 >> 32);
+            out_low[slot0 - begin] = (uint16_t)v0;
+            if (two) {
+                out_pair[slot1 - begin] = (uint32_t)(v1 >> 32);
+                out_low[slot1 - begin] = (uint16_t)v1;
+            }
+        } else {
+            emit(slot0, (uint32_t)(v0 >> 32), (uint32_t)v0);
+            if (two) emit(slot1, (uint32_t)(v1 >> 32), (uint32_t)v1);
+        }
+    }
+    if (!in_lds) return;
+    __syncthreads();
+    for (int32_t i = tid; i < end - begin; i += NT) emit(begin + i, out_pair[i], out_low[i]);
+}
+
+struct PartitionPlan {
+    int shift, buckets, groups, tile, tiles;
+    int64_t n1;
+    size_t off_counts, off_offs, off_ticket, off_status, off_stage, bytes;
+};
+PartitionPlan plan_partition(int64_t num_pairs, int64_t num_experts) {
+    PartitionPlan p;
+    p.shift = 0;
+    while (((num_experts + (1ll << p.shift) - 1) >> p.shift) > kPartMaxBuckets) ++p.shift;
+    p.buckets = (int)((num_experts + (1ll << p.shift) - 1) >> p.shift);
+    p.tile = partition_tile(num_pairs);
+    p.groups = (int)((num_pairs + p.tile - 1) / p.tile);
+    p.n1 = (int64_t)(p.buckets + 1) * p.groups;
+    p.tiles = (int)((p.n1 + kScanTile - 1) / kScanTile);
+    size_t o = 0;
+    auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
+    p.off_counts = take((size_t)p.n1 * 4);
+    p.off_offs = take((size_t)(p.n1 + 1) * 4);
+    p.off_ticket = take(256);
+    p.off_status = take((size_t)p.tiles * 8);
+    p.off_stage = take((size_t)num_pairs * 8);
+    p.bytes = o;
+    return p;
+}
+
 struct BucketPlan {
     int tiles;
     size_t off_cursor, off_ticket, off_status, bytes;
@@ -223,6 +391,44 @@ BucketPlan plan_bucket(int64_t num_experts) {
 }  // namespace
 
 size_t bucket_workspace_bytes(int64_t num_experts) { return plan_bucket(num_experts).bytes; }
+
+// With millions of pairs the partition passes are far ahead of the atomics; with fewer both are a handful of launches
+// at their floor, and below 65536 pairs the tiles would be too few to fill the chip.
+bool bucket_partition_pays(int64_t num_pairs, int64_t num_experts) {
+    if (num_pairs < (1ll << 16) || num_pairs >= (1ll << 31) || num_experts >= (1ll << 31) - 1) return false;
+    const PartitionPlan p = plan_partition(num_pairs, num_experts);
+    return p.shift <= kPartMaxShift && p.n1 < (1ll << 31) - 1;
+}
+
+size_t bucket_partition_workspace_bytes(int64_t num_pairs, int64_t num_experts) {
+    return bucket_partition_pays(num_pairs, num_experts) ? plan_partition(num_pairs, num_experts).bytes : 0;
+}
+
+int bucket_partition(const int64_t* indices, void* workspace, int64_t num_pairs, int64_t num_experts, int top_k,
+                     int32_t* offsets, int32_t* sorted_pairs, uint32_t* tok, uint32_t tok_scale, uint32_t* exp,
+                     uint32_t exp_scale, float* coef_clear, int pack_shift, hipStream_t stream) {
+    const PartitionPlan p = plan_partition(num_pairs, num_experts);
+    char* ws = (char*)workspace;
+    int32_t* counts1 = (int32_t*)(ws + p.off_counts);
+    int32_t* offs1 = (int32_t*)(ws + p.off_offs);
+    int32_t* ticket = (int32_t*)(ws + p.off_ticket);
+    uint64_t* status = (uint64_t*)(ws + p.off_status);
+    uint64_t* stage = (uint64_t*)(ws + p.off_stage);
+    hipLaunchKernelGGL(partition_count_kernel, dim3((unsigned)p.groups), dim3(256), 0, stream, indices, counts1, num_pairs,
+                       num_experts, p.shift, p.buckets, p.groups, p.tile, ticket, status, p.tiles);
+    FMOE_CHECK_LAUNCH("expert bucketing (partition counts)");
+    hipLaunchKernelGGL(bucket_scan_kernel, dim3((unsigned)p.tiles), dim3(kScanThreads), 0, stream, counts1, offs1, p.n1, ticket,
+                       status);
+    FMOE_CHECK_LAUNCH("expert bucketing (partition scan)");
+    hipLaunchKernelGGL(partition_scatter_kernel, dim3((unsigned)p.groups), dim3(256), 0, stream, indices,
+                       (const int32_t*)offs1, stage, coef_clear, num_pairs, num_experts, p.shift, p.buckets, p.groups, p.tile);
+    FMOE_CHECK_LAUNCH("expert bucketing (partition scatter)");
+    hipLaunchKernelGGL(partition_local_kernel, dim3((unsigned)(p.buckets + 1)), dim3(kPartLocalThreads), (size_t)4 << p.shift, stream,
+                       (const uint64_t*)stage, (const int32_t*)offs1, offsets, sorted_pairs, tok, exp, num_experts, p.shift,
+                       p.buckets, p.groups, top_k, tok_scale, exp_scale, pack_shift);
+    FMOE_CHECK_LAUNCH("expert bucketing (partition local)");
+    return FMOE_OK;
+}
 
 int32_t* bucket_counts(void* workspace) { return (int32_t*)workspace; }
 

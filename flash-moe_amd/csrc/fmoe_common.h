@@ -92,6 +92,14 @@ int bucket_scan_fill(const int64_t* indices, void* workspace, int64_t num_pairs,
                      int32_t* offsets, int32_t* sorted_pairs, uint32_t* tok, uint32_t tok_scale, uint32_t* exp,
                      uint32_t exp_scale, float* coef_clear, int pack_shift, int ordered, hipStream_t stream);
 
+// The same grouping without global atomics, by two partition passes (fmoe_bucket.hip), for large numbers of pairs: own
+// workspace, no clear / histogram needed, segments in no particular pair order.  bucket_partition_pays says when to take it.
+bool bucket_partition_pays(int64_t num_pairs, int64_t num_experts);
+size_t bucket_partition_workspace_bytes(int64_t num_pairs, int64_t num_experts);
+int bucket_partition(const int64_t* indices, void* workspace, int64_t num_pairs, int64_t num_experts, int top_k,
+                     int32_t* offsets, int32_t* sorted_pairs, uint32_t* tok, uint32_t tok_scale, uint32_t* exp,
+                     uint32_t exp_scale, float* coef_clear, int pack_shift, hipStream_t stream);
+
 // Plain library GEMM (rocBLAS, loaded on first use) for the operand layouts of the backward passes; row-major
 // C[M,N] = A[M,K] B[K,N] (kBlasNN) or A[K,M]^T B[K,N] (kBlasTN), C = product + beta * C.  Defined in fmoe_mlp_backward.hip.
 enum { kBlasNN = 0, kBlasTN = 1 };

@@ -915,7 +915,7 @@ __global__ __launch_bounds__(kSweepThreads) void expert_states_sweep_kernel(
 struct BucketedPlan {
     int chunk_lanes, num_bands, parts, blocks_per_unit, xcds;
     unsigned grid;
-    size_t off_bucket, off_offsets, off_pairs, off_tok, off_exp, off_a, off_spart, off_xb, off_sweep_keys, off_sweep_coef, bytes;
+    size_t off_bucket, off_part, off_offsets, off_pairs, off_tok, off_exp, off_a, off_spart, off_xb, off_sweep_keys, off_sweep_coef, bytes;
     bool sweep;
 };
 
@@ -949,6 +949,7 @@ BucketedPlan plan_bucketed(int64_t T_, int H, int64_t E, int K, size_t elt) {
     size_t o = 0;
     auto take = [&](size_t n) { const size_t at = o; o = round_up(o + n, 256); return at; };
     p.off_bucket = take(bucket_workspace_bytes(E));
+    p.off_part = take(bucket_partition_workspace_bytes(pairs, E));
     p.off_offsets = take((size_t)(E + 1) * 4);
     p.off_pairs = take((size_t)pairs * 4);
     p.off_tok = take((size_t)pairs * 4);
@@ -988,11 +989,17 @@ int launch_expert_bucketed(int act, const void* x, const void* down, const void*
         // no score phase: the coefficient is the routing weight itself, nothing to group
         return launch_expert_rows<T>(act, x, down, up, indices, gates, T_, H, E, K, out, stream);
     }
-    if (int rc = bucket_clear(ws + p.off_bucket, E, stream)) return rc;
-    if (int rc = bucket_histogram(indices, ws + p.off_bucket, pairs, E, stream)) return rc;
-    if (int rc = bucket_scan_fill(indices, ws + p.off_bucket, pairs, E, K, offsets, sorted_pairs, tokoff, 1u, expoff, 1u, a, 24,
-                                  0, stream))
-        return rc;
+    if (bucket_partition_pays(pairs, E)) {
+        if (int rc = bucket_partition(indices, ws + p.off_part, pairs, E, K, offsets, sorted_pairs, tokoff, 1u, expoff, 1u, a, 24,
+                                      stream))
+            return rc;
+    } else {
+        if (int rc = bucket_clear(ws + p.off_bucket, E, stream)) return rc;
+        if (int rc = bucket_histogram(indices, ws + p.off_bucket, pairs, E, stream)) return rc;
+        if (int rc = bucket_scan_fill(indices, ws + p.off_bucket, pairs, E, K, offsets, sorted_pairs, tokoff, 1u, expoff, 1u, a,
+                                      24, 0, stream))
+            return rc;
+    }
     void* xb = ws + p.off_xb;
     {
         const int64_t packets = T_ * (int64_t)(row_bytes / 16);

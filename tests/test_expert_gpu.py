@@ -206,6 +206,26 @@ def test_expert_out_of_range_ids_contribute_nothing(algo):
     torch.testing.assert_close(got, run(x, wd, wu, idx, g2, algo), rtol=1e-6, atol=1e-8)
 
 
+@pytest.mark.parametrize("E", [1000, 5000, 70000])
+def test_expert_bucketed_grouping_by_partition_with_a_hot_expert_and_invalid_ids(E):
+    """From 65536 pairs on the bucketed schedule groups the pairs with two partition passes (coarse buckets of 1, 8 and 128
+    experts here, the last one partial): one expert chosen six times by every token (12288 pairs: more than a workgroup
+    orders in LDS), ids outside [0, E) in two columns, fp32 against the row schedule and the float64 oracle."""
+    T, H, K = 2048, 128, 32
+    x, wd, wu, idx, g = orc.make_expert_inputs(T, H, E, K, seed=31, std=0.3)
+    idx[:, 0] = 3
+    idx[:, 4:9] = 3
+    idx[::3, 1] = E + 5
+    idx[1::4, 2] = -1
+    idx[:, 3] = E - 1
+    got = run(x, wd, wu, idx, g, "buckets")
+    assert torch.isfinite(got).all() and torch.equal(got, run(x, wd, wu, idx, g, "buckets"))
+    assert rel_fro(got, run(x, wd, wu, idx, g, "rows")) < 2e-6
+    valid = (idx >= 0) & (idx < E)
+    ref = truth64(x, wd, wu, idx.clamp(0, E - 1), g * valid)
+    assert rel_fro(got, ref) < 2e-6
+
+
 def test_expert_empty_and_noncontiguous():
     from flash_moe.ops import flash_expert_func
 
