@@ -52,12 +52,14 @@ int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_k
 bool router_topk_supported(int num_keys, int top_k);
 
 // The fused router (fmoe_router_forward) with the optional row-offset output; defined in fmoe_router_prologue.hip.
+// fixed_scratch: the workspace is the fixed scratch of the no-allocation entry point, which has no room for the normalised
+// copy of x that many tokens would otherwise use.
 int router_forward_impl(const void* x, const void* gate_w, void* running_mean, void* running_var,
                         int64_t* num_batches_tracked, int stats_dtype, int training, float momentum, float eps,
                         int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
                         void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
                         uint32_t* row_offsets, uint32_t row_bytes, void* workspace, size_t workspace_bytes,
-                        hipStream_t stream, int split_query = 0);
+                        hipStream_t stream, int split_query = 0, int fixed_scratch = 0);
 
 // Column-slice schedule of the routed experts on row offsets that are already in place at the start of `workspace`
 // (the layout fmoe_expert_workspace_bytes describes); defined in fmoe_expert.hip.
@@ -77,6 +79,11 @@ int expert_slice_scores(const void* x, const void* table, const uint32_t* off32,
                         int64_t num_experts, int top_k, int dtype, hipStream_t stream);
 int expert_slice_states(const float* coef, const void* table, const uint32_t* off32, void* out, int64_t num_tokens, int hidden,
                         int64_t num_experts, int top_k, int dtype, hipStream_t stream);
+
+// C[M,N] = A[M,K] * B[N,K]^T written in the 16-bit dtype and in fp32, on the shared MLP's tiled kernel (fmoe_mlp.hip);
+// usable when the extents are whole tiles and there are enough of them.
+bool gemm_nt_dual_usable(int64_t M, int N, int K);
+int gemm_nt_dual(const void* A, const void* B, void* C, float* C32, int M, int N, int K, int dtype, hipStream_t stream);
 
 // Expert-centric bucketing (fmoe_bucket.hip): pairs grouped by expert id.  The workspace holds the per-expert counts
 // (bucket_counts; cleared by bucket_clear, filled by bucket_histogram or by a caller's own kernel) and the scan state.

@@ -31,7 +31,7 @@ constexpr int kGemmThreads = 256;
 constexpr int BK = kTileK;        // k extent of a register-staged LDS tile (elements)
 constexpr int kChunksPerRow = kTileChunks;
 
-enum Epilogue { kEpiSwiGLU = 0, kEpiPlain = 1 };
+enum Epilogue { kEpiSwiGLU = 0, kEpiPlain = 1, kEpiDual = 2 };   // Dual: the product in T and, through R, in fp32
 template <bool B> struct Flag { static constexpr bool value = B; };
 
 template <typename T, int BM, int BN, int EPI>
@@ -426,6 +426,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
                     for (int v = 0; v < 16; ++v)
                         store_elem(((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T),
                                    silu(acc[i][j][v]) * acc[i][j + NF / 2][v]);
+        } else if (EPI == kEpiDual) {
+            // R points at an fp32 [M, N] buffer that receives the unrounded sums next to the rounded ones in C
+            float* out32 = reinterpret_cast<float*>(const_cast<T*>(R));
+            const int64_t span_f = ((int64_t)M * N - wave_off) * 4;
+            const int span32_f = (int)(span_f < 0 ? 0 : (span_f < 0x7FFFFFFFll ? span_f : 0x7FFFFFFFll));
+            auto f_rsrc = __builtin_amdgcn_make_buffer_rsrc(out32 + wave_off, 0, span32_f, 0x00020000);
+            const int lane_bytes_f = ((4 * fhalf) * N + frow) * 4;
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+                for (int j = 0; j < NF; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int at = (i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32;
+                        const float sum = acc[i][j][v];      // a scalar copy: the bit cast below must not see a vector element
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, sum), f_rsrc, lane_bytes_f, at * 4, 0);
+                        store_elem(at * (int)sizeof(T), sum);
+                    }
         } else {
             auto r_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(R != nullptr ? R + wave_off : C), 0,
                                                             R != nullptr ? span32 : 0, 0x00020000);   // no residual: reads give 0
@@ -601,6 +619,27 @@ int down_tiled(const void* h, const void* wd, int M, int H, int I, const void* r
     FMOE_CHECK_LAUNCH("fmoe_mlp(down)");
     return FMOE_OK;
 }
+
+}  // namespace
+
+// C[M,N] = A[M,K] * B[N,K]^T in the 16-bit dtype and in fp32 (the same sums before rounding), on 256 x 256 tiles of the
+// DMA kernel: for products large enough to give every compute unit a tile (the router's gate product for tens of thousands
+// of tokens).  The k order of the sums is that of every other kernel here: ascending, 16 values per matrix instruction.
+bool gemm_nt_dual_usable(int64_t M, int N, int K) {
+    return M > 0 && M < (1ll << 31) && N % 256 == 0 && K % 64 == 0 && ((M + 255) / 256) * (int64_t)(N / 256) >= chip_info().cus;
+}
+int gemm_nt_dual(const void* A, const void* B, void* C, float* C32, int M, int N, int K, int dtype, hipStream_t stream) {
+    if (dtype == FMOE_BF16)
+        launch_gemm_dma<bf16_t, 256, 256, 2, 4, 64, 2, kEpiDual, 1>((const bf16_t*)A, (const bf16_t*)B, nullptr, (bf16_t*)C,
+                                                                    (const bf16_t*)C32, M, N, K, stream);
+    else
+        launch_gemm_dma<f16_t, 256, 256, 2, 4, 64, 2, kEpiDual, 1>((const f16_t*)A, (const f16_t*)B, nullptr, (f16_t*)C,
+                                                                   (const f16_t*)C32, M, N, K, stream);
+    FMOE_CHECK_LAUNCH("gate product (tiled)");
+    return FMOE_OK;
+}
+
+namespace {
 
 int check_mlp_shape(const char* who, int64_t T_, int H, int I, int dtype) {
     FMOE_REQUIRE(dtype_ok(dtype), FMOE_ERR_BAD_DTYPE, "%s: unknown dtype %d", who, dtype);

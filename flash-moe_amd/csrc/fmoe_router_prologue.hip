@@ -618,9 +618,27 @@ __global__ __launch_bounds__(256) void router_gate_f32_kernel(const float* __res
         }
 }
 
+// q = round_T((x - mean) * rstd), 16 bytes per thread: the normalised activations as a stand-alone batch-norm emits them,
+// for the gate product on the shared MLP's tiled kernel (many tokens).  mean_rstd: [2][hidden].
+template <typename T>
+__global__ __launch_bounds__(256) void bn_apply_kernel(const u32x4_t* __restrict__ x, const float* __restrict__ mean_rstd,
+                                                       u32x4_t* __restrict__ q, int64_t packets, int hidden) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= packets) return;
+    const int col = (int)(i % (hidden / 8)) * 8;
+    float m8[8], r8[8];
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+        m8[v] = mean_rstd[col + v];
+        r8[v] = mean_rstd[hidden + col + v];
+    }
+    q[i] = normalise16<T>(x[i], m8, r8);
+}
+
 struct ProloguePlan {
     int row_blocks, rows_per_block;
-    size_t off_partial, off_mean_rstd, bytes;
+    size_t off_partial, off_mean_rstd, off_q, base_bytes, bytes;
+    bool tiled_gate;     // enough tokens for the gate product to run on 256 x 256 tiles from a normalised copy of x
 };
 
 ProloguePlan plan_prologue(int64_t T_, int H, int nk) {
@@ -631,8 +649,11 @@ ProloguePlan plan_prologue(int64_t T_, int H, int nk) {
     p.row_blocks = (int)((T_ + p.rows_per_block - 1) / p.rows_per_block);
     p.off_partial = 0;
     p.off_mean_rstd = round_up((size_t)kMaxRowBlocks * 3 * (size_t)H * 4, 256);
-    (void)nk;
-    p.bytes = round_up(p.off_mean_rstd + 2 * (size_t)H * 4, 256);
+    p.base_bytes = round_up(p.off_mean_rstd + 2 * (size_t)H * 4, 256);
+    // the normalised copy (16-bit activations; callers whose workspace stops at base_bytes keep the 64 x 64 gate kernel)
+    p.tiled_gate = gemm_nt_dual_usable(T_, 2 * nk, H);
+    p.off_q = p.base_bytes;
+    p.bytes = p.base_bytes + (p.tiled_gate ? round_up((size_t)T_ * (size_t)H * 2, 256) : 0);
     return p;
 }
 
@@ -1003,7 +1024,7 @@ extern "C" int fmoe_router_forward_noalloc(const void* x, const void* gate_w, vo
     if (int rc = static_scratch(&ws)) return rc;
     return router_forward_impl(x, gate_w, running_mean, running_var, num_batches_tracked, stats_dtype, training, momentum,
                                eps, num_tokens, hidden, num_keys, top_k, dtype, norm_topk_prob, router_logits, logits_fp32,
-                               scores, indices, gates, nullptr, 0u, ws, (size_t)FMOE_NOALLOC_SCRATCH_BYTES, (hipStream_t)stream);
+                               scores, indices, gates, nullptr, 0u, ws, (size_t)FMOE_NOALLOC_SCRATCH_BYTES, (hipStream_t)stream, 0, 1);
 }
 
 int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_mean, void* running_var,
@@ -1011,7 +1032,7 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
                               int64_t num_tokens, int hidden, int num_keys, int top_k, int dtype, int norm_topk_prob,
                               void* router_logits, float* logits_fp32, float* scores, int64_t* indices, void* gates,
                               uint32_t* row_offsets, uint32_t row_bytes, void* workspace, size_t workspace_bytes,
-                              hipStream_t s, int split_query) {
+                              hipStream_t s, int split_query, int fixed_scratch) {
     using namespace fmoe;
     FMOE_REQUIRE(!split_query || (num_keys % 64 == 0 && hidden % 2 == 0), FMOE_ERR_UNSUPPORTED,
                  "fmoe_router_forward_split: num_keys=%d must be a multiple of 64 and hidden=%d even", num_keys, hidden);
@@ -1039,8 +1060,12 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
                  "fmoe_router_forward: hidden=%d must be a multiple of %d and tensors 16-byte aligned", hidden,
                  split_query ? 2 * vec : vec);
     const ProloguePlan p = plan_prologue(num_tokens, hidden, num_keys);
-    FMOE_REQUIRE(workspace_bytes >= p.bytes && aligned16(workspace), FMOE_ERR_WORKSPACE,
-                 "fmoe_router_forward: workspace of %zu bytes needed, %zu given", p.bytes, workspace_bytes);
+    // a workspace without room for the normalised copy (the fixed scratch of the no-allocation entry point) takes the
+    // 64 x 64 gate kernel: the same sums in the same order
+    const bool tiled_gate = p.tiled_gate && dtype != FMOE_F32 && !split_query && !fixed_scratch;
+    const size_t need = fixed_scratch ? p.base_bytes : p.bytes;
+    FMOE_REQUIRE(workspace_bytes >= need && aligned16(workspace), FMOE_ERR_WORKSPACE,
+                 "fmoe_router_forward: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     char* ws = (char*)workspace;
     float* partial = (float*)(ws + p.off_partial);
     float* mean_rstd = (float*)(ws + p.off_mean_rstd);
@@ -1083,6 +1108,22 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
                 default: launch_finalize<f16_t>(partial, p, hidden, training, momentum, eps, running_mean, running_var, num_batches_tracked, mean_rstd, s); break;
             }
             FMOE_CHECK_LAUNCH("fmoe_router_forward(finalize)");
+        }
+        if (tiled_gate) {
+            // fold is false here (at least one 256 x 256 tile per compute unit): mean and 1/std are in the workspace
+            void* q = ws + p.off_q;
+            const int64_t packets = num_tokens * (int64_t)(hidden / 8);
+            if (dtype == FMOE_BF16)
+                hipLaunchKernelGGL((bn_apply_kernel<bf16_t>), dim3((unsigned)((packets + 255) / 256)), dim3(256), 0, s,
+                                   (const u32x4_t*)x, (const float*)mean_rstd, (u32x4_t*)q, packets, hidden);
+            else
+                hipLaunchKernelGGL((bn_apply_kernel<f16_t>), dim3((unsigned)((packets + 255) / 256)), dim3(256), 0, s,
+                                   (const u32x4_t*)x, (const float*)mean_rstd, (u32x4_t*)q, packets, hidden);
+            FMOE_CHECK_LAUNCH("fmoe_router_forward(normalise)");
+            if (int rc = gemm_nt_dual(q, gate_w, router_logits, logits32, M, N, hidden, dtype, s)) return rc;
+            if (top_k == 0) return FMOE_OK;
+            return launch_router_from_logits(logits32, num_tokens, num_keys, top_k, scores, indices, gates, dtype, norm_topk_prob,
+                                             row_offsets, row_bytes, s);
         }
         GateStats st;
         st.ready = fold ? 0 : 1;

@@ -52,6 +52,23 @@ def test_noalloc_router_equals_the_workspace_entry_point_on_two_calls(dtype, tra
         assert int(got[3].min()) >= 0 and int(got[3].max()) < nk * nk
 
 
+@pytest.mark.parametrize("dtype,training", [(torch.bfloat16, True), (torch.float16, False)])
+def test_noalloc_router_equals_the_workspace_entry_point_where_that_one_takes_the_tiled_gate_product(dtype, training):
+    """With at least one 256 x 256 tile of logits per compute unit the workspace entry point normalises x into its workspace
+    and runs the gate product on the shared MLP's tiled kernel; the no-allocation entry point has no room for that copy and
+    keeps the 64 x 64 gate kernel.  Both add the products in ascending k, 16 per matrix instruction: bit-identical."""
+    T, H, nk, K = 16384, 256, 512, 16
+    L = _C.lib()
+    assert L.fmoe_router_workspace_bytes(T, H, nk) >= T * H * 2 > L.fmoe_router_workspace_bytes(T // 2, H, nk)
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn(T, H, generator=g) * 1.3 + 0.2).to(dtype).cuda()
+    w = (torch.randn(2 * nk, H, generator=g) * 0.05).to(dtype).cuda()
+    got = _route("noalloc", x, w, nk, K, training, False)
+    ref = _route("workspace", x, w, nk, K, training, False)
+    for a, b, name in zip(got, ref, ("logits", "logits32", "scores", "indices", "gates", "mean", "var", "count")):
+        assert torch.equal(a, b), f"{name} differs"
+
+
 def test_noalloc_router_rejects_sizes_beyond_its_scratch():
     L = _C.lib()
     x = torch.zeros(4, 4096, device="cuda", dtype=torch.bfloat16)
