@@ -92,7 +92,9 @@ int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, in
  *   gates          [T, top_k]    dtype   out: routing weights (NULL to skip)
  * The normalised activations are rounded to dtype as a stand-alone batch-norm emits them; the product with gate_w,
  * the log-softmax and the pair sums are fp32.  With T == 1 in training mode the call is rejected like
- * nn.BatchNorm1d rejects it.  workspace: fmoe_router_workspace_bytes() bytes, 256-byte aligned.
+ * nn.BatchNorm1d rejects it.  workspace: fmoe_router_workspace_bytes() bytes, 256-byte aligned (batch statistics, mean and
+ * 1/std, and - when the logits give every compute unit a 256 x 256 tile - T*H*2 bytes for the normalised activations, from
+ * which the gate product then runs on the shared MLP's tiled kernel; the logits are the same bit for bit either way).
  * Limits of this build: num_keys <= 32767, top_k as in fmoe_router_topk, num_tokens < 2^31 (FMOE_ERR_UNSUPPORTED beyond); hidden a whole
  * number of 16-byte packets (FMOE_ERR_ALIGNMENT) and, for the 16-bit dtypes, hidden <= 8192.
  */
