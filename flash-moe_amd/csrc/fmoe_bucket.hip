@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kOrderWaves* kWave) void bucket_order_kernel(
     const int64_t* __restrict__ indices, const int32_t* __restrict__ offsets, int32_t* __restrict__ sorted_pairs,
     uint32_t* __restrict__ tok, int64_t num_pairs, int64_t num_experts, int top_k, uint32_t tok_scale) {
     __shared__ uint32_t keys[kOrderLds];
-    __shared__ int32_t wave_count[kOrderWaves];
+    __shared__ int32_t wave_count[4][kOrderWaves];
     const int tid = (int)threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int64_t e_first = (int64_t)blockIdx.x * kOrderWaves;
     {
@@ -182,24 +182,38 @@ __global__ __launch_bounds__(kOrderWaves* kWave) void bucket_order_kernel(
                 if (tok != nullptr) tok[begin + i] = (keys[i] / (uint32_t)top_k) * tok_scale;
             }
         } else {
+            // kOrderBatch rounds of 256 pairs per pair of barriers: their index loads are in flight together
+            constexpr int kOrderBatch = 4, kRound = kOrderWaves * kWave;
             int32_t written = 0;
-            for (int64_t base = 0; base < num_pairs; base += kOrderWaves * kWave) {
-                const int64_t p = base + tid;
-                const bool hit = p < num_pairs && indices[p] == e;
-                const uint64_t ballot = __ballot(hit);
-                if (lane == 0) wave_count[wave] = __popcll(ballot);
+            for (int64_t base = 0; base < num_pairs; base += kOrderBatch * kRound) {
+                bool hit[kOrderBatch];
+                uint64_t ballot[kOrderBatch];
+#pragma unroll
+                for (int u = 0; u < kOrderBatch; ++u) {
+                    const int64_t p = base + u * kRound + tid;
+                    hit[u] = p < num_pairs && indices[p] == e;
+                }
+#pragma unroll
+                for (int u = 0; u < kOrderBatch; ++u) {
+                    ballot[u] = __ballot(hit[u]);
+                    if (lane == 0) wave_count[u][wave] = __popcll(ballot[u]);
+                }
                 __syncthreads();
-                int32_t before = written, all = 0;
-                for (int v = 0; v < kOrderWaves; ++v) {
-                    if (v < wave) before += wave_count[v];
-                    all += wave_count[v];
+#pragma unroll
+                for (int u = 0; u < kOrderBatch; ++u) {
+                    int32_t before = written, all = 0;
+                    for (int v = 0; v < kOrderWaves; ++v) {
+                        if (v < wave) before += wave_count[u][v];
+                        all += wave_count[u][v];
+                    }
+                    if (hit[u]) {
+                        const int64_t p = base + u * kRound + tid;
+                        const int32_t slot = begin + before + __popcll(ballot[u] & ((1ull << lane) - 1ull));
+                        sorted_pairs[slot] = (int32_t)p;
+                        if (tok != nullptr) tok[slot] = (uint32_t)(p / top_k) * tok_scale;
+                    }
+                    written += all;
                 }
-                if (hit) {
-                    const int32_t slot = begin + before + __popcll(ballot & ((1ull << lane) - 1ull));
-                    sorted_pairs[slot] = (int32_t)p;
-                    if (tok != nullptr) tok[slot] = (uint32_t)(p / top_k) * tok_scale;
-                }
-                written += all;
                 __syncthreads();
             }
         }
