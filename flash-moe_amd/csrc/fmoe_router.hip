@@ -584,6 +584,147 @@ __global__ __launch_bounds__(kBigThreads) void router_topk_big_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// top_k up to 4096 with any num_keys (what the kernel above cannot hold in LDS): one workgroup per token.  Neither a half
+// (up to 65535 keys) nor the candidate list (sum_i floor(K/i), 35 000 for K = 4096) is stored: the K-th largest 64-bit key of
+// a list is found by radix selection (eight passes over the list, a 256-bin histogram in LDS per pass; the list is
+// regenerated from global memory or from the sorted halves each time), the K keys at or above it are collected and
+// bitonic-sorted in LDS.  Same pruning, same keys (unique: they carry the index), so the same result as the other
+// kernels, ties to the lowest flat index.  A completeness path: milliseconds for thousands of tokens.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int kRadixMaxTopK = 4096;
+
+// K-th largest of the keys `each(f)` feeds to f (every thread its share; the same keys on every call), by the whole
+// workgroup.  hist: 256 counters; pick: two words.
+template <typename Each>
+__device__ inline uint64_t block_kth_largest(Each each, int want, uint32_t* hist, uint64_t* pick) {
+    uint64_t prefix = 0ull;
+    int remaining = want;
+    for (int d = 7; d >= 0; --d) {
+        for (int i = (int)threadIdx.x; i < 256; i += (int)blockDim.x) hist[i] = 0u;
+        __syncthreads();
+        each([&](uint64_t key) {
+            if (d == 7 || (key >> (8 * (d + 1))) == prefix) atomicAdd(&hist[(uint32_t)(key >> (8 * d)) & 255u], 1u);
+        });
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int above = 0, digit = 0;
+            for (int bin = 255; bin >= 0; --bin) {
+                const int n = (int)hist[bin];
+                if (above + n >= remaining) {
+                    digit = bin;
+                    break;
+                }
+                above += n;
+            }
+            pick[0] = prefix << 8 | (uint64_t)digit;
+            pick[1] = (uint64_t)(remaining - above);
+        }
+        __syncthreads();
+        prefix = pick[0];
+        remaining = (int)pick[1];
+    }
+    return prefix;
+}
+
+template <typename T, typename TG, bool FROM_LOGITS>
+__global__ __launch_bounds__(kBigThreads) void router_topk_radix_kernel(
+    const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, T* __restrict__ scores, int64_t* __restrict__ indices,
+    TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets, uint32_t row_bytes) {
+    __shared__ uint64_t keys[kRadixMaxTopK];
+    __shared__ float half_score[2][kRadixMaxTopK];
+    __shared__ uint32_t half_index[2][kRadixMaxTopK];
+    __shared__ uint32_t hist[256];
+    __shared__ uint64_t pick[2];
+    __shared__ float stat[2];
+    __shared__ int filled;
+    const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    int m = 64;
+    while (m < top_k) m <<= 1;
+    // keys at or above `tau` into keys[0..top_k), the rest of keys[0..m) zero, sorted descending
+    auto collect_and_sort = [&](auto each, uint64_t tau) {
+        for (int i = tid; i < m; i += kBigThreads) keys[i] = 0ull;
+        if (tid == 0) filled = 0;
+        __syncthreads();
+        each([&](uint64_t key) {
+            if (key >= tau) {
+                const int at = atomicAdd(&filled, 1);
+                if (at < top_k) keys[at] = key;
+            }
+        });
+        __syncthreads();
+        block_sort_desc(keys, m);
+    };
+    for (int64_t token = blockIdx.x; token < num_tokens; token += gridDim.x) {
+        for (int h = 0; h < 2; ++h) {
+            const T* row = FROM_LOGITS ? lp + (token * 2 + h) * nk : lp + ((int64_t)h * num_tokens + token) * nk;
+            if (FROM_LOGITS) {
+                // by one wave, in the order the one-wave-per-token kernels use: identical log-probabilities
+                if (tid < kWave) {
+                    float mx = -INFINITY;
+                    for (int p = lane; p < nk; p += kWave) mx = fmaxf(mx, Elem<T>::to_f32(row[p]));
+                    mx = wave_max(mx);
+                    float se = 0.0f;
+                    for (int p = lane; p < nk; p += kWave) se += expf(Elem<T>::to_f32(row[p]) - mx);
+                    const float lse = logf(wave_sum(se));
+                    if (lane == 0) {
+                        stat[0] = mx;
+                        stat[1] = lse;
+                    }
+                }
+                __syncthreads();
+            }
+            const float shift = FROM_LOGITS ? stat[0] : 0.0f, lse = FROM_LOGITS ? stat[1] : 0.0f;
+            auto each_key = [&](auto f) {
+                for (int p = tid; p < nk; p += kBigThreads) {
+                    const float v = Elem<T>::to_f32(row[p]);
+                    f(make_key(FROM_LOGITS ? (v - shift) - lse : v, (uint32_t)p));
+                }
+            };
+            const uint64_t tau = block_kth_largest(each_key, top_k, hist, pick);
+            collect_and_sort(each_key, tau);
+            for (int r = tid; r < top_k; r += kBigThreads) {
+                half_score[h][r] = key_score(keys[r]);
+                half_index[h][r] = key_index(keys[r]);
+            }
+            __syncthreads();
+        }
+        // candidates: rank i of half 0 with ranks 0 .. top_k/(i+1)-1 of half 1; a wave per row, lanes along the row
+        auto each_candidate = [&](auto f) {
+            for (int i = wave; i < top_k; i += kBigThreads / kWave) {
+                const int n = top_k / (i + 1);
+                const float si = half_score[0][i];
+                const uint32_t base = half_index[0][i] * (uint32_t)nk;
+                for (int j = lane; j < n; j += kWave) f(make_key(round_through<T>(si + half_score[1][j]), base + half_index[1][j]));
+            }
+        };
+        const uint64_t tau = block_kth_largest(each_candidate, top_k, hist, pick);
+        collect_and_sort(each_candidate, tau);
+        if (tid < kWave) {
+            float total = 0.0f;
+            if (gates != nullptr && norm_topk_prob) {
+                for (int p = lane; p < top_k; p += kWave) total += expf(key_score(keys[p]));
+                total = wave_sum(total);
+            }
+            stat[0] = total;
+        }
+        __syncthreads();
+        const float total = stat[0];
+        for (int p = tid; p < top_k; p += kBigThreads) {
+            const uint64_t key = keys[p];
+            const int64_t o = token * top_k + p;
+            scores[o] = Elem<T>::from_f32(key_score(key));
+            indices[o] = (int64_t)key_index(key);
+            if (row_offsets != nullptr) row_offsets[o] = key_index(key) * row_bytes;
+            if (gates != nullptr) {
+                const float e = expf(key_score(key));
+                gates[o] = Elem<TG>::from_f32(norm_topk_prob ? e / total : e);
+            }
+        }
+        __syncthreads();
+    }
+}
+
 int count_candidates(int top_k) {
     int n = 0;
     for (int i = 1; i <= top_k; ++i) n += top_k / i;
@@ -598,8 +739,15 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
     const int64_t max_blocks = (int64_t)chip_info().cus * 8;   // a few resident blocks per CU; the kernel loops over tokens
     const dim3 grid((unsigned)(blocks_needed < max_blocks ? blocks_needed : max_blocks));
     const dim3 block(kRouterWaves * kWave);
-    if (K > kMaxTopK) {      // the workgroup-per-token kernel; its limits are checked by the callers
+    if (K > kMaxTopK) {      // the workgroup-per-token kernels; their limits are checked by the callers
         const int64_t big_blocks = T_ < (int64_t)chip_info().cus * 2 ? T_ : (int64_t)chip_info().cus * 2;
+        if (K > kBigMaxTopK || nk > kBigMaxKeys) {
+            const int64_t radix_blocks = T_ < (int64_t)chip_info().cus ? T_ : (int64_t)chip_info().cus;
+            hipLaunchKernelGGL((router_topk_radix_kernel<T, TG, FROM_LOGITS>), dim3((unsigned)radix_blocks), dim3(kBigThreads), 0,
+                               stream, (const T*)lp, T_, nk, K, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes);
+            FMOE_CHECK_LAUNCH("fmoe_router_topk");
+            return FMOE_OK;
+        }
         hipLaunchKernelGGL((router_topk_big_kernel<T, TG, FROM_LOGITS>), dim3((unsigned)big_blocks), dim3(kBigThreads), 0, stream,
                            (const T*)lp, T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes);
         FMOE_CHECK_LAUNCH("fmoe_router_topk");
@@ -643,7 +791,7 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
 }  // namespace
 
 bool router_topk_supported(int num_keys, int top_k) {
-    return top_k <= kMaxTopK || (top_k <= kBigMaxTopK && num_keys <= kBigMaxKeys);
+    return top_k <= kRadixMaxTopK;       // <= 256: a wave per token; beyond: a workgroup per token
 }
 
 int launch_router_from_logits(const float* logits, int64_t num_tokens, int num_keys, int top_k, float* scores,
@@ -669,8 +817,7 @@ extern "C" int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int n
                  "num_experts_per_tok should be in [0, %d], but got %d", num_keys, top_k);
     FMOE_REQUIRE(num_keys <= 65535, FMOE_ERR_UNSUPPORTED, "fmoe_router_topk: num_keys=%d > 65535", num_keys);
     FMOE_REQUIRE(router_topk_supported(num_keys, top_k), FMOE_ERR_UNSUPPORTED,
-                 "fmoe_router_topk: top_k=%d > %d needs top_k <= %d and num_keys <= %d (num_keys=%d)", top_k, kMaxTopK, kBigMaxTopK,
-                 kBigMaxKeys, num_keys);
+                 "fmoe_router_topk: top_k=%d > %d (num_keys=%d)", top_k, kRadixMaxTopK, num_keys);
     if (num_tokens == 0 || top_k == 0) return FMOE_OK;
     FMOE_REQUIRE(log_probs && scores && indices, FMOE_ERR_NULL_POINTER, "fmoe_router_topk: null tensor pointer");
     hipStream_t s = (hipStream_t)stream;

@@ -67,9 +67,9 @@ const char* fmoe_last_error(void);
  *   gates      [num_tokens, top_k]        dtype      optional (NULL to skip): exp(score), divided by the
  *                                                    per-token sum when norm_topk_prob != 0
  * Requires 0 <= top_k <= num_keys (same rule as the reference's assert).
- * Limits of this build (FMOE_ERR_UNSUPPORTED beyond): num_keys <= 65535; top_k <= 256, or top_k <= 1024 with
- * num_keys <= 8192 (a slower workgroup-per-token kernel).  The reference accepts any top_k <= num_keys
- * (flash_router.py:261-263).
+ * Limits of this build (FMOE_ERR_UNSUPPORTED beyond): num_keys <= 65535; top_k <= 4096 (beyond 256 a workgroup per
+ * token: in-LDS sorts up to top_k 1024 with num_keys <= 8192, radix selection otherwise - milliseconds for thousands of
+ * tokens).  The reference accepts any top_k <= num_keys (flash_router.py:261-263); its own benchmarks stop at 4096.
  */
 int fmoe_router_topk(const void* log_probs, int64_t num_tokens, int num_keys, int top_k, int dtype,
                      void* scores, int64_t* indices, void* gates, int norm_topk_prob, void* stream);
@@ -244,7 +244,7 @@ int fmoe_mlp_down(const void* act, const void* down_w, int64_t num_tokens, int h
  *   running_mean / running_var / num_batches_tracked, stats_dtype, training, momentum, eps: as in fmoe_router_forward
  *   out [T,H] dtype; router_logits [T,2*nk] dtype
  *   indices_out [T,K] int64 and gates_out [T,K] dtype: optional (NULL keeps them in the workspace)
- * Requires nk*nk <= E and 0 <= top_k <= nk.  The limits of the three stages apply (top_k <= 256 or <= 1024 with nk <= 8192, nk <= 32767, the expert
+ * Requires nk*nk <= E and 0 <= top_k <= nk.  The limits of the three stages apply (top_k <= 4096, nk <= 32767, the expert
  * schedules' limits above; hidden and intermediate multiples of 8 for the 16-bit dtypes), and T, E < 2^31.
  */
 size_t fmoe_block_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int num_keys, int64_t num_experts,

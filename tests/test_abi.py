@@ -56,8 +56,8 @@ def test_router_argument_checks():
     assert lib.fmoe_router_topk(a, 4, 8, 4, 7, a, a, None, 0, None) == -4          # dtype
     assert lib.fmoe_router_topk(a, -1, 8, 4, _C.F32, a, a, None, 0, None) == -2     # shape
     assert lib.fmoe_router_topk(None, 4, 8, 4, _C.F32, a, a, None, 0, None) == -1   # null
-    assert lib.fmoe_router_topk(a, 4, 2048, 1025, _C.F32, a, a, None, 0, None) == -5  # top_k > 1024
-    assert lib.fmoe_router_topk(a, 4, 9000, 300, _C.F32, a, a, None, 0, None) == -5   # top_k > 256 needs num_keys <= 8192
+    assert lib.fmoe_router_topk(a, 4, 8192, 4097, _C.F32, a, a, None, 0, None) == -5  # top_k > 4096
+    assert lib.fmoe_router_topk(a, 4, 70000, 4, _C.F32, a, a, None, 0, None) == -5    # num_keys > 65535
     # empty problems succeed without a launch
     assert lib.fmoe_router_topk(None, 0, 8, 4, _C.F32, None, None, None, 0, None) == 0
     assert lib.fmoe_router_topk(a, 4, 8, 0, _C.F32, a, a, None, 0, None) == 0

@@ -59,6 +59,8 @@ def check_fp32_case(lp, nk, K):
     (200, 128, 128), (150, 512, 64), (40, 300, 100), (64, 600, 64), (48, 520, 128),
     # top_k beyond 256, up to num_keys as the reference allows (flash_router.py:261-263): the workgroup-per-token kernel
     (24, 512, 512), (20, 300, 257), (12, 1024, 1000), (600, 400, 320),
+    # beyond what sorts in LDS (top_k > 1024, or > 256 with more than 8192 keys): radix selection, up to top_k 4096
+    (5, 2048, 1500), (3, 9000, 300), (2, 4096, 4096), (40, 1100, 1100),
 ])
 def test_router_fp32_log_probs(T, nk, K):
     check_fp32_case(orc.make_router_inputs(T, nk, seed=T + nk), nk, K)
@@ -123,9 +125,7 @@ def test_router_limits_of_the_large_top_k_kernel():
     from flash_moe.ops import flash_router_func
 
     with pytest.raises(ValueError, match="top_k"):
-        flash_router_func(torch.zeros(2, 2, 2048, device="cuda"), 2048, 1025)          # beyond 1024
-    with pytest.raises(ValueError, match="top_k"):
-        flash_router_func(torch.zeros(2, 2, 9000, device="cuda"), 9000, 300)           # beyond 256 needs num_keys <= 8192
+        flash_router_func(torch.zeros(2, 2, 8192, device="cuda"), 8192, 4097)          # beyond 4096
 
 
 def test_router_noncontiguous_input_and_empty():
@@ -161,7 +161,8 @@ def _fused(x, wr, nk, K, norm_flag, dtype, training=True, rm=None, rv=None):
 
 
 @pytest.mark.parametrize("T,H,nk,K", [(512, 256, 32, 16), (1000, 1024, 128, 64), (130, 72, 100, 37), (64, 2048, 512, 128),
-                                      (40, 256, 320, 300)])
+                                      (40, 256, 320, 300),
+                                      (24, 128, 1200, 1100)])     # top_k beyond 1024: the radix-selection kernel, from logits
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_fused_router_matches_oracle_prologue(T, H, nk, K, dtype):
     g = torch.Generator().manual_seed(T + nk)
