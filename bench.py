@@ -17,6 +17,7 @@ that is already resident in HBM.  The last line printed is one JSON object:
   router_c2      the routing stage alone on the router benchmark shape: module semantics (every half scores the full
                  query) and the configuration as worded (two sub-key tables on the two halves of the query)
   block_c5       the largest block (32768 tokens, 262144 experts), with its stages and the expert op's roofline entry
+  block_c1       the reference's CPU-runnable configuration (fp32, 512 tokens, 1024 experts) on the GPU, next to cpu_baseline_c1
   mlp_fp32       the shared MLP of the same shape in fp32 (v_mfma_f32_32x32x2_f32) against the dense fp32 matrix peak
   cpu_baseline   the CPU restatement of the reference's eager path (oracle/) on the same block, timed on
                  this machine's host cores; cpu_baseline_c1 / cpu_baseline_c4_fp32: the reference's own CPU
@@ -371,6 +372,20 @@ def bench_block_c5(dtype, iters):
                 mlp_TFLOPs=round(6 * T * cfg["hidden"] * cfg["inter"] / ((times["mlp_gate_up"] + times["mlp_down"]) * 1e-3) / 1e12, 1))
 
 
+def bench_block_c1(iters):
+    """The reference's own CPU-runnable configuration (fp32, 512 tokens, 1024 experts, top-16) on the GPU: launch-bound."""
+    import torch
+
+    m, x = synthetic_block(C1, torch.float32, "cuda:0")
+    T = C1["batch"] * C1["seq"]
+    with torch.no_grad():
+        per_call = event_times_ms(lambda: m(x), iters, warmup=5)
+    ms = statistics.median(per_call)
+    return dict(workload=f"C1 full block: fp32, {T} tokens, hidden {C1['hidden']}, intermediate {C1['inter']}, "
+                         f"{C1['experts']} experts, top-{C1['top_k']}, train-mode batch norm",
+                ms_per_step=round(ms, 4), step_us=spread(per_call), tokens_per_s=round(T / (ms * 1e-3)))
+
+
 def bench_mlp_fp32(iters):
     """The C4 shared MLP in fp32: both GEMMs on v_mfma_f32_32x32x2_f32, priced against the dense fp32 matrix peak."""
     import torch
@@ -589,6 +604,8 @@ def main():
         result["block_c5"] = bench_block_c5(dtype, 5)
         log("block C5:", result["block_c5"])
         torch.cuda.empty_cache()
+        result["block_c1"] = bench_block_c1(50)
+        log("block C1:", result["block_c1"])
         result["mlp_fp32"] = result["rooflines_all"]["mlp_fp32"] = bench_mlp_fp32(10)
         log("mlp fp32:", result["mlp_fp32"])
         result["backward_c4"] = bench_backward_c4(dtype, 10)

@@ -35,6 +35,36 @@ template <> struct Mfma32<float> {
 };
 template <typename T> constexpr int kMfmaPerRun = sizeof(T) == 4 ? 4 : 1;   // matrix instructions per Mfma32<T>::run
 
+// v_mfma_f32_16x16x32_{bf16,f16}: D[16x16] += A[16x32] * B[32x16].  Lane l supplies row l%16 of A (column l%16 of B) and 8
+// consecutive k values chosen by l/16; it receives D[4*(l/16) + v][l%16] in register v (four registers).  Under the power
+// limit the chip sustains about 12 % more multiply-adds with this shape than with 32x32x16 on random data.
+template <typename T> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+    using Frag = bf16x8_t;
+    __device__ static f32x4_t run(Frag a, Frag b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Mfma16<f16_t> {
+    using Frag = f16x8_t;
+    __device__ static f32x4_t run(Frag a, Frag b, f32x4_t c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+
+// What the tiled kernel needs to know about a fragment shape: FR = rows (and columns) of a fragment, kChunks = 16-byte
+// pieces of a row one k-step consumes (lane l reads piece l / FR of its row l % FR), Acc with kAccRegs registers, register
+// v of lane l holding D[8*(v/4) + 4*(l/FR) + v%4][l % FR] (both shapes).
+template <typename T, int FR> struct MfmaShape;
+template <typename T> struct MfmaShape<T, 32> {
+    using Frag = typename Mfma32<T>::Frag;
+    using Acc = f32x16_t;
+    static constexpr int kChunks = 2, kAccRegs = 16, kInstr = kMfmaPerRun<T>;
+    __device__ static Acc run(Frag a, Frag b, Acc c) { return Mfma32<T>::run(a, b, c); }
+};
+template <typename T> struct MfmaShape<T, 16> {
+    using Frag = typename Mfma16<T>::Frag;
+    using Acc = f32x4_t;
+    static constexpr int kChunks = 4, kAccRegs = 4, kInstr = 1;
+    __device__ static Acc run(Frag a, Frag b, Acc c) { return Mfma16<T>::run(a, b, c); }
+};
+
 // Register-staged LDS tiles: rows of 64 elements (128 bytes), 16-byte chunk index XOR-ed with (row & 7).
 constexpr int kTileK = 64;
 constexpr int kTileChunks = kTileK / 8;

@@ -1,8 +1,8 @@
 // Shared SwiGLU MLP for gfx950:  out = (silu(x Wg^T) * (x Wu^T)) Wd^T [+ residual]
 //
 // Two launches of one MFMA GEMM  C[M,N] = A[M,K] * B[N,K]^T  (both operands K-contiguous, which is how x, the
-// nn.Linear weights and the [T,I] activation are laid out, so a lane's 8 consecutive k values for
-// v_mfma_f32_32x32x16 are one 16-byte LDS read):
+// nn.Linear weights and the [T,I] activation are laid out, so a lane's 8 consecutive k values for one matrix
+// instruction are one 16-byte LDS read):
 //   1. gate/up: the B tile holds BN/2 rows of Wg and the same BN/2 rows of Wu, so each wave owns matching gate
 //      and up accumulators and the epilogue writes silu(gate)*up, rounded once, to the [T,I] workspace.  The gate
 //      and up products never go to memory.
@@ -10,8 +10,8 @@
 //
 // Main kernel (gemm_dma_kernel), used when the extents are multiples of the tile: tiles go global -> LDS
 // directly (global_load_lds_dwordx4, no staging registers) into NSTAGE LDS stages, issued NSTAGE-1 k-tiles
-// ahead of their use; one workgroup barrier per k-tile; 32x32x16 MFMA fragments are read with 16-byte
-// ds_reads.  An LDS row is one k-tile of one matrix row; its 16-byte chunks are XOR-swizzled with a key built
+// ahead of their use; one workgroup barrier per k-tile; MFMA fragments (v_mfma_f32_16x16x32 for the 16-bit types) are
+// read with 16-byte ds_reads.  An LDS row is one k-tile of one matrix row; its 16-byte chunks are XOR-swizzled with a key built
 // from the row index so that the 16 lanes the 256-byte-per-clock LDS serves per cycle hit 64 different banks.
 // Because a DMA load writes 64 consecutive chunks, the swizzle is applied on the global side: each lane fetches
 // the chunk that belongs at its LDS position.  Workgroup ids are remapped so that each XCD (ids are dealt
@@ -193,19 +193,27 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(
 // ------------------------------------------------------------------------------------------------------------
 // LDS-DMA pipelined kernel.  WAVES_M x WAVES_N waves, each (BM/WAVES_M) x (BN/WAVES_N); BKT = k extent of a stage.
 // ------------------------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
+// FR: fragment shape (32: v_mfma_f32_32x32x16 / 32x32x2; 16: v_mfma_f32_16x16x32).  SPLIT: a k-step's A fragments are read and
+// multiplied in SPLIT parts (its B fragments stay for the whole k-step), which halves the registers the read-ahead needs.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF, int FR = 32, int SPLIT = 1>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     const T* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1, T* __restrict__ C,
     const T* __restrict__ R, int M, int N, int K, int tiles_m, int tiles_n, int xcds) {
-    using Frag = typename Mfma32<T>::Frag;
+    using Shape = MfmaShape<T, FR>;
+    using Frag = typename Shape::Frag;
+    using Acc = typename Shape::Acc;
+    constexpr int NV = Shape::kAccRegs;
     constexpr int NWAVES = WAVES_M * WAVES_N;
-    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MF = WM / 32, NF = WN / 32;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MF = WM / FR, NF = WN / FR;
     constexpr int EPC = 16 / (int)sizeof(T);        // elements per 16-byte chunk
     constexpr int CPR = BKT / EPC;                  // 16-byte chunks per LDS row
     constexpr int RPI = 64 / CPR;                   // rows one wave-wide DMA load covers
     constexpr int ROWS_PER_IT = NWAVES * RPI;       // rows all waves cover per DMA round
     constexpr int STAGE = (BM + BN) * BKT;          // elements per stage
-    constexpr int KSTEPS = BKT / (2 * EPC);         // a k-step is 32 bytes of a row: one chunk per lane half
+    constexpr int KSTEPS = BKT / (Shape::kChunks * EPC);   // a k-step is kChunks 16-byte pieces of a row: one per lane group
+    constexpr int SPK = KSTEPS * SPLIT;             // steps (a part of a k-step's A fragments against all its B fragments) per k-tile
+    constexpr int MFS = MF / SPLIT;
+    static_assert(MF % SPLIT == 0 && WM % FR == 0 && WN % FR == 0, "fragments tile the wave tile");
     constexpr int ROW_SHIFT = (CPR == 8) ? 1 : 2;   // log2(rows per 256 bytes)
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
     constexpr int A_ROUNDS = BM / ROWS_PER_IT, B_ROUNDS = BN / ROWS_PER_IT;
@@ -270,22 +278,22 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         }
     };
 
-    // Fragment rows of a lane are (multiple of 32) + frow: the swizzle key is the same for all of them, so the
+    // Fragment rows of a lane are (multiple of FR) + frow: the swizzle key is the same for all of them, so the
     // address is (row base + one per-k-step offset) + an immediate per fragment.
-    const int frow = lane & 31, fhalf = lane >> 5;
+    const int frow = lane % FR, fhalf = lane / FR;       // fhalf: which 16-byte piece of a k-step the lane supplies
     const int key_f = (frow >> ROW_SHIFT) & (CPR - 1);
     const int a_row_bytes = (wm * WM + frow) * BKT * (int)sizeof(T);
     int b_row_bytes[NF];
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
         int row;
-        if (EPI == kEpiSwiGLU) row = (j < NF / 2) ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - NF / 2) * 32;
-        else row = wn * WN + j * 32;
+        if (EPI == kEpiSwiGLU) row = (j < NF / 2) ? wn * (WN / 2) + j * FR : BN / 2 + wn * (WN / 2) + (j - NF / 2) * FR;
+        else row = wn * WN + j * FR;
         b_row_bytes[j] = (BM + row + frow) * BKT * (int)sizeof(T);
     }
     int pc[KSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) pc[ks] = ((ks * 2 + fhalf) ^ key_f) << 4;
+    for (int ks = 0; ks < KSTEPS; ++ks) pc[ks] = ((ks * Shape::kChunks + fhalf) ^ key_f) << 4;
 
     const int k_tiles = K / BKT;
     int tile = (int)blockIdx.x;
@@ -295,18 +303,25 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
     for (int s = 0; s < NSTAGE - 1; ++s)
         if (s < k_tiles) issue(s, lds + s * STAGE);
 
-    // Fragments of k-step ks+PF are read from LDS while the MFMAs of k-step ks run (PF+1 register buffers); the
-    // read-ahead crosses k-tile boundaries, so the barrier that publishes the next stage sits PF k-steps before the
-    // end of a k-tile and the matrix pipe always has work queued while a wave waits.
+    // Fragments of step q+PF are read from LDS while the MFMAs of step q run (PF+1 register buffers for the A parts; B
+    // fragments are read with the first part of their k-step); the read-ahead crosses k-tile boundaries, so the barrier
+    // that publishes the next stage sits PF steps before the end of a k-tile and the matrix pipe always has work queued
+    // while a wave waits.
     constexpr int RING = PF + 1;
-    static_assert(KSTEPS % RING == 0 && PF >= 1 && PF < KSTEPS + 1, "fragment buffers rotate with period RING");
-    Frag fa[RING][MF], fb[RING][NF];
-    auto read_frags = [&](const char* stage, int ks, Frag (&a)[MF], Frag (&b)[NF]) {
+    constexpr int RINGB = SPLIT == 1 ? RING : 2;
+    static_assert(SPK % RING == 0 && PF >= 1 && PF < SPK + 1, "fragment buffers rotate with period RING");
+    static_assert(SPLIT == 1 || (PF <= SPLIT && KSTEPS % 2 == 0), "with split k-steps at most the next k-step's B fragments are in flight");
+    Frag fa[RING][MFS], fb[RINGB][NF];
+    auto b_slot = [](int q) { return SPLIT == 1 ? q % RING : (q / SPLIT) % 2; };     // q: step inside the k-tile (may exceed SPK by PF)
+    auto read_frags = [&](const char* stage, int q, Frag (&a)[MFS], Frag (&b)[NF]) {
+        const int ks = q / SPLIT, part = q % SPLIT;
 #pragma unroll
-        for (int i = 0; i < MF; ++i)
-            a[i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + i * 32 * BKT * (int)sizeof(T));
+        for (int i = 0; i < MFS; ++i)
+            a[i] = *reinterpret_cast<const Frag*>(stage + a_row_bytes + pc[ks] + (part * MFS + i) * FR * BKT * (int)sizeof(T));
+        if (part == 0) {
 #pragma unroll
-        for (int j = 0; j < NF; ++j) b[j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
+            for (int j = 0; j < NF; ++j) b[j] = *reinterpret_cast<const Frag*>(stage + b_row_bytes[j] + pc[ks]);
+        }
     };
     // Entering k-tile kt (kt = 0: from the tile prologue): my share of its stage has landed once at most the loads of
     // the NSTAGE-2 younger k-tiles are outstanding; my reads of the stage that is overwritten next are complete (all
@@ -320,17 +335,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         if (kt + NSTAGE - 1 < k_tiles) issue(kt + NSTAGE - 1, lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE);
     };
     while (true) {
-        f32x16_t acc[MF][NF];
+        Acc acc[MF][NF];
 #pragma unroll
         for (int i = 0; i < MF; ++i)
 #pragma unroll
             for (int j = 0; j < NF; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+                for (int v = 0; v < NV; ++v) acc[i][j][v] = 0.0f;
 
         enter_k_tile(0);
 #pragma unroll
-        for (int s = 0; s < PF; ++s) read_frags(reinterpret_cast<const char*>(lds), s, fa[s], fb[s]);
+        for (int s = 0; s < PF; ++s) read_frags(reinterpret_cast<const char*>(lds), s, fa[s % RING], fb[b_slot(s)]);
         // the last k-tile has no successor to read ahead into: it is a separate copy of the body, so that no branch
         // merges a path with reads in flight into the MFMA sequence
         auto k_tile_body = [&](int kt, auto last_tag) {
@@ -338,30 +353,33 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
             const char* stage = reinterpret_cast<const char*>(lds + (kt % NSTAGE) * STAGE);
             const char* next_stage = reinterpret_cast<const char*>(lds + ((kt + 1) % NSTAGE) * STAGE);
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                constexpr int kReads = MF + NF, kMfmas = MF * NF;     // kMfmas runs of kMfmaPerRun<T> instructions
-                const int nxt = ks + PF;
-                const bool reads = nxt < KSTEPS || !kLast;
+            for (int q = 0; q < SPK; ++q) {
+                const int nxt = q + PF;
+                constexpr int kMfmas = MFS * NF;     // runs of Shape::kInstr instructions
+                const bool reads = nxt < SPK || !kLast;
+                const int n_reads = MFS + ((nxt % SPLIT) == 0 ? NF : 0);
                 __builtin_amdgcn_sched_barrier(0);
-                if (nxt < KSTEPS) {
-                    read_frags(stage, nxt, fa[nxt % RING], fb[nxt % RING]);
+                if (nxt < SPK) {
+                    read_frags(stage, nxt, fa[nxt % RING], fb[b_slot(nxt)]);
                 } else if (!kLast) {
-                    if (nxt == KSTEPS) {
+                    if (nxt == SPK) {
                         enter_k_tile(kt + 1);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    read_frags(next_stage, nxt - KSTEPS, fa[nxt % RING], fb[nxt % RING]);
+                    read_frags(next_stage, nxt - SPK, fa[nxt % RING], fb[b_slot(nxt)]);
                 }
+                const int part = q % SPLIT;
 #pragma unroll
-                for (int i = 0; i < MF; ++i)
+                for (int i = 0; i < MFS; ++i)
 #pragma unroll
-                    for (int j = 0; j < NF; ++j) acc[i][j] = Mfma32<T>::run(fa[ks % RING][i], fb[ks % RING][j], acc[i][j]);
+                    for (int j = 0; j < NF; ++j)
+                        acc[part * MFS + i][j] = Shape::run(fa[q % RING][i], fb[b_slot(q)][j], acc[part * MFS + i][j]);
                 // issue order: the LDS reads spread evenly behind the MFMAs
-                constexpr int kPer = (kReads + kMfmas - 1) / kMfmas;
+                constexpr int kPer = (MFS + NF + kMfmas - 1) / kMfmas;
 #pragma unroll
-                for (int q = 0; q < kMfmas; ++q) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerRun<T>, 0);
-                    if (reads && q * kPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
+                for (int m = 0; m < kMfmas; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, Shape::kInstr, 0);
+                    if (reads && m * kPer < n_reads) __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);
                 }
             }
         };
@@ -380,8 +398,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
                 if (s < k_tiles) issue(s, lds + s * STAGE);
         }
 
-        // D fragment layout of v_mfma_f32_32x32x*: lane l, register v holds
-        //   row = 8*(v/4) + 4*(l/32) + (v%4)   (A / M index),   col = l%32   (B / N index)
+        // D fragment layout (both shapes): lane l, register v holds
+        //   row = 8*(v/4) + 4*(l/FR) + (v%4)   (A / M index),   col = l%FR   (B / N index)
         // Buffer addressing: a wave-uniform descriptor of the rows from the wave's first one on, a scalar byte offset
         // per (fragment, register) and one 32-bit byte offset per lane - no vector address arithmetic per element.
         const int lane_bytes = ((4 * fhalf) * N + frow) * (int)sizeof(T);
@@ -401,6 +419,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
         auto store_elem = [&](int uni_bytes, float value) { store_to(c_rsrc, uni_bytes, value); };
         // 16-bit outputs round once, so the fast reciprocal's last-bit error is invisible; fp32 divides
         auto silu = [](float v) { return sizeof(T) == 4 ? silu_f32(v) : silu_fast_f32(v); };
+        // element offset of (fragment i, fragment column j, register v) from the wave's first output element
+        auto elem_at = [&](int i, int j, int v) { return (i * FR + 8 * (v / 4) + (v % 4)) * N + j * FR; };
         if (EPI == kEpiSwiGLU) {
             if (R != nullptr) {
                 // keep the gate and up products for a backward pass: planes [0] and [1] of a [2, M, N] buffer
@@ -412,8 +432,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                     for (int j = 0; j < NF / 2; ++j)
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int uni = ((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T);
+                        for (int v = 0; v < NV; ++v) {
+                            const int uni = elem_at(i, j, v) * (int)sizeof(T);
                             store_to(g_rsrc, uni, acc[i][j][v]);
                             store_to(u_rsrc, uni, acc[i][j + NF / 2][v]);
                         }
@@ -423,9 +443,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                 for (int j = 0; j < NF / 2; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        store_elem(((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T),
-                                   silu(acc[i][j][v]) * acc[i][j + NF / 2][v]);
+                    for (int v = 0; v < NV; ++v)
+                        store_elem(elem_at(i, j, v) * (int)sizeof(T), silu(acc[i][j][v]) * acc[i][j + NF / 2][v]);
         } else if (EPI == kEpiDual) {
             // R points at an fp32 [M, N] buffer that receives the unrounded sums next to the rounded ones in C
             float* out32 = reinterpret_cast<float*>(const_cast<T*>(R));
@@ -438,8 +457,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
 #pragma unroll
                 for (int j = 0; j < NF; ++j)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int at = (i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32;
+                    for (int v = 0; v < NV; ++v) {
+                        const int at = elem_at(i, j, v);
                         const float sum = acc[i][j][v];      // a scalar copy: the bit cast below must not see a vector element
                         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, sum), f_rsrc, lane_bytes_f, at * 4, 0);
                         store_elem(at * (int)sizeof(T), sum);
@@ -451,10 +470,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
             for (int i = 0; i < MF; ++i)
 #pragma unroll
                 for (int j = 0; j < NF; ++j) {
-                    float res[16];
+                    float res[NV];
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int uni = ((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T);
+                    for (int v = 0; v < NV; ++v) {
+                        const int uni = elem_at(i, j, v) * (int)sizeof(T);
                         if constexpr (sizeof(T) == 4) {
                             res[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r_rsrc, lane_bytes, uni, 0));
                         } else {
@@ -463,8 +482,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_dma_kernel(
                         }
                     }
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        store_elem(((i * 32 + 8 * (v / 4) + (v % 4)) * N + j * 32) * (int)sizeof(T), acc[i][j][v] + res[v]);
+                    for (int v = 0; v < NV; ++v) store_elem(elem_at(i, j, v) * (int)sizeof(T), acc[i][j][v] + res[v]);
                 }
         }
         if (next >= num_tiles) break;
@@ -539,7 +557,7 @@ void launch_gemm(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, 
                        stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n, chip_info().xcds);
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int BKT, int NSTAGE, int EPI, int PF, int FR = 32, int SPLIT = 1>
 void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
     constexpr int BN_OUT = (EPI == kEpiSwiGLU) ? BN / 2 : BN;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = N / BN_OUT;      // a ragged last row of tiles is allowed
@@ -550,12 +568,18 @@ void launch_gemm_dma(const T* A, const T* B0, const T* B1, T* C, const T* R, int
     const ChipInfo& chip = chip_info();
     const int resident = chip.cus * kPerCu;
     const int grid = total < resident ? total : resident;
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI, PF>), dim3((unsigned)grid),
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, WAVES_M, WAVES_N, BKT, NSTAGE, EPI, PF, FR, SPLIT>), dim3((unsigned)grid),
                        dim3(WAVES_M * WAVES_N * 64), 0, stream, A, B0, B1, C, R, M, N, K, tiles_m, tiles_n, chip.xcds);
 }
 
 // k extent of one LDS stage of the DMA kernel: 128 bytes of a row for every element type
 template <typename T> constexpr int kStageK = 128 / (int)sizeof(T);
+// 16-bit products run on v_mfma_f32_16x16x32 (more multiply-adds per joule than 32x32x16, which is what bounds these
+// kernels); a k-step is then half a stage, so the read-ahead is one step, and the 256 x 256 tile reads a k-step's A
+// fragments in four parts to stay inside 256 registers per wave (in two parts it spills 24).  fp32 keeps 32x32x2.
+template <typename T> constexpr int kFragRows = sizeof(T) == 2 ? 16 : 32;
+template <typename T> constexpr int kBigSplit = sizeof(T) == 2 ? 4 : 1;
+template <typename T> constexpr int kSmallAhead = sizeof(T) == 2 ? 1 : 3;
 
 // Ragged shapes: the bounds-checked kernels (register-staged MFMA for 16-bit, FMA for fp32).
 template <typename T, int EPI>
@@ -567,14 +591,14 @@ void launch_ragged(const T* A, const T* B0, const T* B1, T* C, const T* R, int M
 }
 
 // Tile choice: 256-wide tiles (8 waves, two per SIMD) halve the L2 -> LDS traffic per MFMA but need one per CU to
-// occupy the chip; otherwise 128x128 tiles of 4 waves, which read a whole k-tile of fragments ahead (PF = 3): one
+// occupy the chip; otherwise 128x128 tiles of 4 waves, which read half a k-tile of fragments ahead (a whole one in fp32): one
 // workgroup per CU with four stages in flight when every tile gets a CU of its own, two per CU with two stages else.
 template <typename T, int EPI>
 void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, int64_t tiles,
                         hipStream_t stream) {
     constexpr int KT = kStageK<T>;
-    if (tiles <= chip_info().cus) launch_gemm_dma<T, 128, 128, 2, 2, KT, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
-    else launch_gemm_dma<T, 128, 128, 2, 2, KT, 2, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+    if (tiles <= chip_info().cus) launch_gemm_dma<T, 128, 128, 2, 2, KT, 4, EPI, kSmallAhead<T>, kFragRows<T>>(A, B0, B1, C, R, M, N, K, stream);
+    else launch_gemm_dma<T, 128, 128, 2, 2, KT, 2, EPI, kSmallAhead<T>, kFragRows<T>>(A, B0, B1, C, R, M, N, K, stream);
 }
 
 // Few tokens: 64-row tiles (wave tiles of 32 x 64 or 32 x 32), so that a batch of a few hundred tokens still gives
@@ -582,9 +606,9 @@ void launch_small_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, 
 template <typename T, int EPI>
 void launch_narrow_tiles(const T* A, const T* B0, const T* B1, T* C, const T* R, int M, int N, int K, hipStream_t stream) {
     if (EPI == kEpiPlain && (int64_t)((M + 63) / 64) * (N / 128) < chip_info().cus && N % 64 == 0)
-        launch_gemm_dma<T, 64, 64, 2, 2, kStageK<T>, 4, kEpiPlain, 3>(A, B0, B1, C, R, M, N, K, stream);
+        launch_gemm_dma<T, 64, 64, 2, 2, kStageK<T>, 4, kEpiPlain, kSmallAhead<T>, kFragRows<T>>(A, B0, B1, C, R, M, N, K, stream);
     else
-        launch_gemm_dma<T, 64, 128, 2, 2, kStageK<T>, 4, EPI, 3>(A, B0, B1, C, R, M, N, K, stream);
+        launch_gemm_dma<T, 64, 128, 2, 2, kStageK<T>, 4, EPI, kSmallAhead<T>, kFragRows<T>>(A, B0, B1, C, R, M, N, K, stream);
 }
 
 template <typename T>
@@ -593,7 +617,7 @@ int gate_up_tiled(const void* x, const void* wg, const void* wu, int M, int H, i
     // the DMA kernel moves 16-byte pieces (fp32 callers need not align their tensors; those take the ragged kernel)
     const bool k_ok = H % kStageK<T> == 0 && aligned16(x) && aligned16(wg) && aligned16(wu);
     if (k_ok && I % 128 == 0 && (int64_t)((M + 255) / 256) * (I / 128) >= chip_info().cus)
-        launch_gemm_dma<T, 256, 256, 2, 4, kStageK<T>, 2, kEpiSwiGLU, 1>(A, G, U, (T*)h, S, M, I, H, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, kStageK<T>, 2, kEpiSwiGLU, 1, kFragRows<T>, kBigSplit<T>>(A, G, U, (T*)h, S, M, I, H, stream);
     else if (k_ok && I % 64 == 0 && (int64_t)((M + 127) / 128) * (I / 64) >= chip_info().cus)
         launch_small_tiles<T, kEpiSwiGLU>(A, G, U, (T*)h, S, M, I, H, (int64_t)((M + 127) / 128) * (I / 64), stream);
     else if (k_ok && I % 64 == 0)
@@ -609,7 +633,7 @@ int down_tiled(const void* h, const void* wd, int M, int H, int I, const void* r
     const T *A = (const T*)h, *W = (const T*)wd, *R = (const T*)residual;
     const bool k_ok = I % kStageK<T> == 0 && aligned16(h) && aligned16(wd);
     if (k_ok && H % 256 == 0 && (int64_t)((M + 255) / 256) * (H / 256) >= chip_info().cus)
-        launch_gemm_dma<T, 256, 256, 2, 4, kStageK<T>, 2, kEpiPlain, 1>(A, W, nullptr, (T*)out, R, M, H, I, stream);
+        launch_gemm_dma<T, 256, 256, 2, 4, kStageK<T>, 2, kEpiPlain, 1, kFragRows<T>, kBigSplit<T>>(A, W, nullptr, (T*)out, R, M, H, I, stream);
     else if (k_ok && H % 128 == 0 && (int64_t)((M + 127) / 128) * (H / 128) >= chip_info().cus)
         launch_small_tiles<T, kEpiPlain>(A, W, nullptr, (T*)out, R, M, H, I, (int64_t)((M + 127) / 128) * (H / 128), stream);
     else if (k_ok && H % 128 == 0)
