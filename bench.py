@@ -188,8 +188,8 @@ def stage_kernels(m, x):
 LAUNCHES = {
     "router_forward": ["bn_block_stats_kernel", "router_gate_kernel", "router_select_kernel"],
     "router_topk": ["router_select_kernel"],
-    "expert": ["expert_prepare_kernel", "expert_scores_slice_kernel", "expert_gate_kernel", "expert_states_slice_kernel"],
-    "expert_c5": ["bucket_clear_kernel", "bucket_histogram_kernel", "bucket_scan_kernel", "bucket_fill_kernel",
+    "expert": ["expert_scores_slice_kernel", "expert_gate_kernel", "expert_states_slice_kernel"],
+    "expert_c5": ["partition_count_kernel", "bucket_scan_kernel", "partition_scatter_kernel", "partition_local_kernel",
                   "expert_band_copy_kernel", "expert_scores_bucketed_kernel", "expert_gate_sorted_kernel",
                   "expert_owner_sort_kernel", "expert_states_sweep_kernel"],
     "mlp_gate_up": ["gemm_dma_kernel<256x256 tiles, SwiGLU epilogue>"],

@@ -303,11 +303,13 @@ template <int N, int STEP> __device__ inline float transpose_sum(const float (&p
     }
 }
 
-template <typename T, int CL>
+// IDS: the row offsets are not prepared yet: they are taken from the int64 ids (an id outside [0, num_experts) gives the
+// out-of-bounds offset) and the workgroups of slice 0 also store them to off32 for the launches that follow.
+template <typename T, int CL, bool IDS = false>
 __global__ __launch_bounds__(256) void expert_scores_slice_kernel(
     const T* __restrict__ x, const T* __restrict__ down, uint32_t table_bytes, const uint32_t* __restrict__ off32,
     float* __restrict__ spart, int64_t num_tokens, int hidden, int top_k, int num_slices, int blocks_per_slice,
-    int tokens_per_block, int xcds) {
+    int tokens_per_block, int xcds, const int64_t* __restrict__ ids = nullptr, int64_t num_experts = 0) {
     constexpr int V = Elem<T>::kVec;
     constexpr int PPL = kWave / CL;                         // pairs per wave-wide load
     int slice, tb;
@@ -329,7 +331,16 @@ __global__ __launch_bounds__(256) void expert_scores_slice_kernel(
         const uint32_t* tok_off = off32 + t * top_k;
         for (int k0 = 0; k0 < top_k; k0 += kWave) {
             // one coalesced load brings the row offsets of 64 pairs; lane (pg, c) then needs those of pairs u*PPL+pg
-            const uint32_t mine = k0 + lane < top_k ? tok_off[k0 + lane] : kBadOffset;
+            uint32_t mine = kBadOffset;
+            if constexpr (IDS) {
+                if (k0 + lane < top_k) {
+                    const int64_t e = ids[t * top_k + k0 + lane];
+                    if (e >= 0 && e < num_experts) mine = (uint32_t)e * (uint32_t)(hidden * (int)sizeof(T));
+                    if (slice == 0) const_cast<uint32_t*>(tok_off)[k0 + lane] = mine;
+                }
+            } else {
+                if (k0 + lane < top_k) mine = tok_off[k0 + lane];
+            }
             u32x4_t w[CL];
 #pragma unroll
             for (int u = 0; u < CL; ++u) {
@@ -470,19 +481,29 @@ SlicePlan plan_slices(int64_t T_, int H, int64_t E, int K, size_t elt) {
     return p;
 }
 
+// ids != nullptr: off32 is written by this launch (from the ids) instead of read
 template <typename T>
 int launch_slice_scores(const void* x, const void* table, const uint32_t* off32, float* spart, int64_t T_, int H, int64_t E,
-                        int K, hipStream_t stream) {
+                        int K, hipStream_t stream, const int64_t* ids = nullptr) {
     const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
     const uint32_t table_bytes = (uint32_t)(E * (int64_t)H * (int64_t)sizeof(T));
-    if (p.chunk_lanes == 16)
+    if (ids != nullptr) {
+        if (p.chunk_lanes == 16)
+            hipLaunchKernelGGL((expert_scores_slice_kernel<T, 16, true>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
+                               (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
+                               p.tokens_per_block, p.xcds, ids, E);
+        else
+            hipLaunchKernelGGL((expert_scores_slice_kernel<T, 8, true>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
+                               (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
+                               p.tokens_per_block, p.xcds, ids, E);
+    } else if (p.chunk_lanes == 16)
         hipLaunchKernelGGL((expert_scores_slice_kernel<T, 16>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
                            (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
-                           p.tokens_per_block, p.xcds);
+                           p.tokens_per_block, p.xcds, (const int64_t*)nullptr, (int64_t)0);
     else
         hipLaunchKernelGGL((expert_scores_slice_kernel<T, 8>), dim3(p.grid), dim3(256), 0, stream, (const T*)x,
                            (const T*)table, table_bytes, off32, spart, T_, H, K, p.num_slices, p.blocks_per_slice,
-                           p.tokens_per_block, p.xcds);
+                           p.tokens_per_block, p.xcds, (const int64_t*)nullptr, (int64_t)0);
     FMOE_CHECK_LAUNCH("routed experts (slice scores)");
     return FMOE_OK;
 }
@@ -503,9 +524,11 @@ int launch_slice_states(const float* a, const void* table, const uint32_t* off32
 }
 
 // Scores, gate and states launches on row offsets that already sit at the start of the workspace.
+// ids != nullptr: the offsets are not in the workspace yet; the score launch writes them on its way
 template <typename T>
 int launch_expert_slices_prepared(int act, const void* x, const void* down, const void* up, const void* gates, int64_t T_,
-                                  int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+                                  int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream,
+                                  const int64_t* ids = nullptr) {
     const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
     char* ws = (char*)workspace;
     const uint32_t* off32 = (const uint32_t*)(ws + p.off_idx32);
@@ -514,7 +537,7 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
     const int64_t pairs = T_ * K;
     const unsigned flat_grid = (unsigned)((pairs + 255) / 256);
     if (act != kActNone)
-        if (int rc = launch_slice_scores<T>(x, down, off32, spart, T_, H, E, K, stream)) return rc;
+        if (int rc = launch_slice_scores<T>(x, down, off32, spart, T_, H, E, K, stream, ids)) return rc;
     // without a score (product-key memory) the coefficient is the routing weight: no partial sums are read
     if (act == kActSilu)
         hipLaunchKernelGGL((expert_gate_kernel<T, kActSilu>), dim3(flat_grid), dim3(256), 0, stream, (const float*)spart,
@@ -532,6 +555,8 @@ int launch_expert_slices_prepared(int act, const void* x, const void* down, cons
 template <typename T>
 int launch_expert_slices(int act, const void* x, const void* down, const void* up, const int64_t* indices, const void* gates,
                          int64_t T_, int H, int64_t E, int K, void* out, void* workspace, hipStream_t stream) {
+    // with a score phase the score launch turns the ids into row offsets itself (and stores them for the launches after it)
+    if (act != kActNone) return launch_expert_slices_prepared<T>(act, x, down, up, gates, T_, H, E, K, out, workspace, stream, indices);
     const SlicePlan p = plan_slices(T_, H, E, K, sizeof(T));
     uint32_t* off32 = (uint32_t*)((char*)workspace + p.off_idx32);
     const int64_t pairs = T_ * K;
