@@ -89,6 +89,23 @@ def test_mlp_leading_dims_and_residual():
     assert flash_mlp_func(x[:0], wg, wu, wd).shape == (0, 128)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,H,I", [(4096, 1024, 4096), (1024, 1024, 4096), (192, 128, 256), (200, 72, 136)])
+def test_mlp_residual_is_added_in_every_tile_shape_and_dtype(dtype, T, H, I):
+    # the block's "experts + mlp" is the down projection's epilogue: one case per kernel the dispatch can pick (256 x 256 and
+    # 128 x 128 tiles, 64-row tiles, the bounds-checked kernel).  The residual is large against the product, so a lane that
+    # reads a neighbour's residual shows at once; the sum is rounded once, from the fp32 accumulator.
+    from flash_moe.ops.hip.flash_mlp import mlp_forward
+
+    x, wg, wu, wd = make(T, H, I, dtype, seed=T + H)
+    res = torch.randn(T, H, generator=torch.Generator().manual_seed(5)).to(dtype)
+    got = mlp_forward(*cuda(x, wg, wu, wd), residual=res.cuda()).cpu()
+    ref64 = truth64(x, wg, wu, wd) + res.double()
+    assert got.dtype == dtype and got.shape == (T, H)
+    assert rel_fro(got, ref64) < {torch.float32: 2e-6, torch.bfloat16: 6e-3, torch.float16: 8e-4}[dtype]
+    assert (got.double() - ref64).abs().max() < {torch.float32: 1e-5, torch.bfloat16: 4e-2, torch.float16: 6e-3}[dtype]
+
+
 def test_mlp_linearity_full_size():
     # C4 at full size: out is linear in the down projection and in the up projection
     from flash_moe.ops import flash_mlp_func
