@@ -92,7 +92,10 @@ def mlp_backward(dout, x, gate_weight, up_weight, down_weight, saved=None):
     code = _C.dtype_code(x.dtype)
     if saved is not None and (saved.shape != (2, num_tokens, inter) or saved.dtype != x.dtype or not saved.is_contiguous()):
         raise ValueError("saved must be the contiguous [2, T, I] tensor mlp_forward_saving returned")
-    dx, dwg, dwu, dwd = torch.empty_like(x2), torch.empty_like(wg), torch.empty_like(wu), torch.empty_like(wd)
+    # the two [I, H] gradients sit behind each other in one buffer: the library then forms them as one [2I, H] product
+    dwgu = torch.empty((2 * inter, hidden), device=wg.device, dtype=wg.dtype)
+    dwg, dwu = dwgu[:inter], dwgu[inter:]
+    dx, dwd = torch.empty_like(x2), torch.empty_like(wd)
     if num_tokens == 0:
         return dx.view(x.shape), dwg.zero_(), dwu.zero_(), dwd.zero_()
     L = _C.lib()

@@ -408,6 +408,48 @@ def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
         assert rel_fro(a, b) < (1e-6 if dtype == torch.float32 else 2e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("stacked_weights", [False, True])
+@pytest.mark.parametrize("stacked_grads", [False, True])
+def test_mlp_backward_with_adjacent_and_separate_buffers(dtype, stacked_weights, stacked_grads):
+    # fmoe_mlp_backward forms dWg and dWu as one product when dup_w starts where dgate_w ends, and dx as one product when
+    # up_w starts where gate_w ends; with separate buffers it makes two calls each.  Every combination against float64.
+    from flash_moe import _C
+
+    T, H, I = 320, 256, 384
+    x = torch.randn(T, H, generator=gen(1)).to(dtype)
+    wg, wu, wd = ((torch.randn(s, generator=gen(k)) * 0.05).to(dtype) for k, s in ((2, (I, H)), (3, (I, H)), (4, (H, I))))
+    dy = torch.randn(T, H, generator=gen(5)).to(dtype)
+    ref_leaves = [t.double().requires_grad_(True) for t in (x, wg, wu, wd)]
+    orc.mlp_forward(*ref_leaves).backward(dy.double())
+
+    xg, dyg, wdg = x.cuda(), dy.cuda(), wd.cuda()
+    if stacked_weights:
+        w2 = torch.cat([wg, wu]).cuda()
+        wgg, wug = w2[:I], w2[I:]
+        assert wug.data_ptr() == wgg.data_ptr() + I * H * wgg.element_size()
+    else:
+        w2 = torch.empty(2 * I * H + 64, device="cuda", dtype=dtype)          # a gap of 64 elements between the two
+        wgg, wug = w2[:I * H].view(I, H).copy_(wg), w2[I * H + 64:].view(I, H).copy_(wu)
+    if stacked_grads:
+        g2 = torch.empty(2 * I, H, device="cuda", dtype=dtype)
+        dwg, dwu = g2[:I], g2[I:]
+    else:
+        g2 = torch.empty(2 * I * H + 64, device="cuda", dtype=dtype)
+        dwg, dwu = g2[:I * H].view(I, H), g2[I * H + 64:].view(I, H)
+    dx, dwd = torch.empty_like(xg), torch.empty_like(wdg)
+    L, code = _C.lib(), _C.dtype_code(dtype)
+    ws_bytes = L.fmoe_mlp_backward_workspace_bytes(T, H, I, code)
+    ws = torch.empty(ws_bytes, device="cuda", dtype=torch.uint8)
+    status = L.fmoe_mlp_backward(_C.ptr(dyg), _C.ptr(xg), _C.ptr(wgg), _C.ptr(wug), _C.ptr(wdg), None, T, H, I, code, _C.ptr(dx),
+                                 _C.ptr(dwg), _C.ptr(dwu), _C.ptr(dwd), _C.ptr(ws), ws_bytes, _C.current_stream(xg.device))
+    _C.check(status, "fmoe_mlp_backward")
+    torch.cuda.synchronize()
+    for name, got, ref in zip(("dx", "dgate", "dup", "ddown"), (dx, dwg, dwu, dwd), ref_leaves):
+        fro = rel_fro(got.cpu(), ref.grad)
+        assert fro < GRAD_FRO[dtype], f"{name}: relative Frobenius error {fro:.3e}"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("training", [True, False])
 @pytest.mark.parametrize("T,H,nk", [(256, 128, 16), (1000, 1024, 128), (65, 64, 8), (256, 128, 32), (1024, 1024, 128),
