@@ -226,6 +226,35 @@ def test_expert_bucketed_grouping_by_partition_with_a_hot_expert_and_invalid_ids
     assert rel_fro(got, ref) < 2e-6
 
 
+def test_expert_bucketed_grouping_with_the_largest_coarse_buckets():
+    """Six million experts (rows of 128 bytes): the partition passes use coarse buckets of 2^13 experts, whose counters
+    fill 32 KiB of a workgroup's LDS, and the second phase is the row kernel (the table is beyond the sweep's key range).
+    Against the row schedule on the GPU and, for a sample of tokens, the float64 oracle on the rows those tokens use."""
+    from flash_moe.ops.hip.flash_expert import expert_forward
+
+    T, H, E, K = 2048, 64, 6_000_000, 32
+    g0 = torch.Generator(device="cuda").manual_seed(5)
+    x = (torch.randn(T, H, device="cuda", generator=g0) * 0.5).bfloat16()
+    wd = (torch.randn(E, H, device="cuda", generator=g0) * 0.3).bfloat16()
+    wu = (torch.randn(E, H, device="cuda", generator=g0) * 0.3).bfloat16()
+    idx = torch.randint(0, E, (T, K), device="cuda", generator=g0)
+    idx[:, 0] = E - 1                      # the last (partial) coarse bucket, chosen by every token
+    idx[::5, 1] = E                        # out of range
+    idx[:, 2] = idx[:, 3]                  # duplicates add
+    g = torch.rand(T, K, device="cuda", generator=g0).bfloat16()
+    got = expert_forward(x, wd, wu, idx, g, algo=ALGOS["buckets"])
+    assert torch.isfinite(got).all() and torch.equal(got, expert_forward(x, wd, wu, idx, g, algo=ALGOS["buckets"]))
+    rows = expert_forward(x, wd, wu, idx, g, algo=ALGOS["rows"])
+    assert rel_fro(got.cpu(), rows.cpu()) < 4e-3
+    sample = torch.arange(0, T, 97, device="cuda")
+    ids = idx[sample]
+    valid = (ids >= 0) & (ids < E)
+    used, inverse = torch.unique(ids.clamp(0, E - 1), return_inverse=True)
+    ref = orc.expert_forward(x[sample].double().cpu(), wd[used].double().cpu(), wu[used].double().cpu(), inverse.cpu(),
+                             (g[sample].double() * valid).cpu())
+    assert rel_fro(got[sample].cpu(), ref) < 4e-3
+
+
 def test_expert_empty_and_noncontiguous():
     from flash_moe.ops import flash_expert_func
 
