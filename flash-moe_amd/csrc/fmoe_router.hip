@@ -364,8 +364,11 @@ __device__ inline void select_topk_sorted(const uint64_t (&key)[R], int k, uint6
 constexpr int kSelectMaxCand = 11 * kWave;
 struct CandidateTable { uint16_t pair[kSelectMaxCand]; };
 
-template <typename T, typename TG, int RK, int RH, int RC, bool FROM_LOGITS>
-__global__ __launch_bounds__(kRouterWaves* kWave) void router_select_kernel(
+// OCC: waves per SIMD the register allocation must leave room for.  With more than four tokens per SIMD eight resident
+// waves (at most 64 registers, a few of them spilled for the larger lists) finish sooner than seven, whose eighth token
+// per SIMD would wait for a second round; with at most four tokens per SIMD the unconstrained allocation is faster.
+template <typename T, typename TG, int RK, int RH, int RC, bool FROM_LOGITS, int OCC>
+__global__ __launch_bounds__(kRouterWaves* kWave, OCC) void router_select_kernel(
     const T* __restrict__ lp, int64_t num_tokens, int nk, int top_k, int num_cand, T* __restrict__ scores,
     int64_t* __restrict__ indices, TG* __restrict__ gates, int norm_topk_prob, uint32_t* __restrict__ row_offsets,
     uint32_t row_bytes, const CandidateTable table) {
@@ -754,9 +757,18 @@ int launch_router(const void* lp, int64_t T_, int nk, int K, void* scores, int64
         return FMOE_OK;
     }
     // lists that fit the registers of a wave take the threshold selection
-#define FMOE_LAUNCH_SELECT(RK_, RH_, RC_)                                                                              \
-    hipLaunchKernelGGL((router_select_kernel<T, TG, RK_, RH_, RC_, FROM_LOGITS>), grid, block, 0, stream, (const T*)lp, \
-                       T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets, row_bytes, table)
+    const bool crowded = T_ > (int64_t)chip_info().cus * 4 * kRouterWaves;      // more than four tokens per SIMD
+#define FMOE_LAUNCH_SELECT(RK_, RH_, RC_)                                                                                    \
+    do {                                                                                                                     \
+        if (crowded)                                                                                                         \
+            hipLaunchKernelGGL((router_select_kernel<T, TG, RK_, RH_, RC_, FROM_LOGITS, 8>), grid, block, 0, stream,         \
+                               (const T*)lp, T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets,        \
+                               row_bytes, table);                                                                            \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((router_select_kernel<T, TG, RK_, RH_, RC_, FROM_LOGITS, 1>), grid, block, 0, stream,         \
+                               (const T*)lp, T_, nk, K, num_cand, (T*)scores, indices, (TG*)gates, norm, row_offsets,        \
+                               row_bytes, table);                                                                            \
+    } while (0)
     CandidateTable table;
     if (K <= 128 && nk <= 512) {
         int c = 0;
