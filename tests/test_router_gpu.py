@@ -57,6 +57,8 @@ def check_fp32_case(lp, nk, K):
     (77, 100, 37), (5, 13, 13), (64, 8, 1), (33, 256, 200), (1, 128, 64), (1030, 64, 64),
     # every top-k kernel variant: lists in registers (nk <= 128 or <= 512, K <= 64 or <= 128) and the group scan beyond
     (200, 128, 128), (150, 512, 64), (40, 300, 100), (64, 600, 64), (48, 520, 128),
+    # more than four tokens per SIMD: the instances compiled for eight waves per SIMD (C2 above is one; C5 in the block tests)
+    (4200, 128, 100), (4200, 320, 48), (4200, 512, 128),
     # top_k beyond 256, up to num_keys as the reference allows (flash_router.py:261-263): the workgroup-per-token kernel
     (24, 512, 512), (20, 300, 257), (12, 1024, 1000), (600, 400, 320),
     # beyond what sorts in LDS (top_k > 1024, or > 256 with more than 8192 keys): radix selection, up to top_k 4096
