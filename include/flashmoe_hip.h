@@ -327,7 +327,7 @@ int fmoe_swiglu_backward(const void* dc, const void* a, const void* b, int64_t r
  * ddown_w [H,I].  saved_products: the [2,T,I] buffer fmoe_mlp_gate_up_save() filled in the forward, or NULL to
  * recompute the gate and up products here.  The transposed-operand GEMMs are rocBLAS calls (loaded on first use;
  * FMOE_ERR_LIBRARY if unavailable).  When dup_w starts where dgate_w ends (one [2I,H] buffer) the two weight gradients
- * are formed as one product, and when up_w starts where gate_w ends so is dx; separate buffers work as well. */
+ * are formed as one product (faster; the sums may differ in the last bit from two products); separate buffers work as well. */
 size_t fmoe_mlp_backward_workspace_bytes(int64_t num_tokens, int hidden, int intermediate, int dtype);
 
 int fmoe_mlp_backward(const void* dy, const void* x, const void* gate_w, const void* up_w, const void* down_w,

@@ -412,8 +412,8 @@ def test_mlp_backward_with_saved_products_equals_recomputation(dtype):
 @pytest.mark.parametrize("stacked_weights", [False, True])
 @pytest.mark.parametrize("stacked_grads", [False, True])
 def test_mlp_backward_with_adjacent_and_separate_buffers(dtype, stacked_weights, stacked_grads):
-    # fmoe_mlp_backward forms dWg and dWu as one product when dup_w starts where dgate_w ends, and dx as one product when
-    # up_w starts where gate_w ends; with separate buffers it makes two calls each.  Every combination against float64.
+    # fmoe_mlp_backward forms dWg and dWu as one product when dup_w starts where dgate_w ends, two otherwise; weights that
+    # happen to follow each other in memory must make no difference.  Every combination against float64.
     from flash_moe import _C
 
     T, H, I = 320, 256, 384
