@@ -1140,17 +1140,21 @@ int fmoe::router_forward_impl(const void* x, const void* gate_w, void* running_m
         st.num_batches_tracked = num_batches_tracked;
         st.mean_rstd = mean_rstd;
         const size_t stats_bytes = (size_t)((hidden + kTileK - 1) / kTileK) * kTileK * 2 * sizeof(float);
-        // few tiles with a long k loop: four k groups per workgroup; many tiles already fill the chip
+        // few tiles with a long k loop: four k groups per workgroup, two for up to two tiles per compute unit; many tiles
+        // already fill the chip
         const bool k_groups = (int64_t)tiles_m * tiles_n <= chip_info().cus && (split_query ? hidden / 2 : hidden) >= 8 * kTileK;
 #define FMOE_LAUNCH_GATE(TT, KG)                                                                                            \
     hipLaunchKernelGGL((router_gate_kernel<TT, KG>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256 * KG), stats_bytes, s,  \
                        (const TT*)x, (const TT*)gate_w, st, logits32, (TT*)router_logits, M, N, hidden, tiles_m, tiles_n,   \
                        split_query, chip_info().xcds)
+        const bool k_pairs = !k_groups && (int64_t)tiles_m * tiles_n <= 2 * chip_info().cus && (split_query ? hidden / 2 : hidden) >= 8 * kTileK;
         if (dtype == FMOE_BF16) {
             if (k_groups) FMOE_LAUNCH_GATE(bf16_t, 4);
+            else if (k_pairs) FMOE_LAUNCH_GATE(bf16_t, 2);
             else FMOE_LAUNCH_GATE(bf16_t, 1);
         } else {
             if (k_groups) FMOE_LAUNCH_GATE(f16_t, 4);
+            else if (k_pairs) FMOE_LAUNCH_GATE(f16_t, 2);
             else FMOE_LAUNCH_GATE(f16_t, 1);
         }
 #undef FMOE_LAUNCH_GATE
